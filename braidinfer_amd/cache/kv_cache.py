@@ -43,10 +43,18 @@ class CacheNeed:
     # read again, pages wholly before it go back to the pool).  None: the window's rule.  Units whose needs
     # are to share a group name the same function object.
     live_from: Optional[Callable[[int], int]] = None
+    # A unit that keeps one row for every `tokens_per_row` tokens (a row of a block's pooled keys and
+    # values, say): a sequence of L tokens holds L // tokens_per_row rows, one for each complete block,
+    # and pages are counted in rows.  Such a unit keeps all its rows (no window, no `live_from`).
+    tokens_per_row: int = 1
 
     @property
     def key_dim(self) -> int:
         return self.head_dim
+
+    def rows_of(self, length: int) -> int:
+        """Rows that a sequence of `length` tokens holds in a unit of this need."""
+        return int(length) // self.tokens_per_row
 
     def first_live(self, length: int) -> int:
         """The first position of a sequence of `length` tokens that a later token may still read."""
@@ -114,6 +122,9 @@ class CacheGroup:
         self._staging = _PinnedStaging(max(4096, 2 * max_pages_per_seq)) if self.device.type == "cuda" else None
         if need.kv_heads <= 0 or need.key_dim <= 0 or need.val_dim < 0:
             raise CacheError(f"a cache unit needs kv heads and a key width above zero, got {need}")
+        if need.tokens_per_row < 1 or (need.tokens_per_row > 1 and (need.window is not None or need.live_from is not None)):
+            raise CacheError(f"a cache unit keeps one row for every tokens_per_row >= 1 tokens, and all of them when "
+                             f"that is more than one, got {need}")
         self.key_elems = need.kv_heads * page_tokens * need.key_dim        # of one page
         self.page_elems = self.key_elems + need.kv_heads * page_tokens * need.val_dim
         self.storage: Dict[int, torch.Tensor] = {}
@@ -140,11 +151,11 @@ class CacheGroup:
 
     # -- bookkeeping, all on the host ------------------------------------------------
     def pages_needed(self, slot: int, new_len: int) -> int:
-        return max(0, -(-new_len // self.page_tokens) - len(self.pages[slot]))
+        return max(0, -(-self.need.rows_of(new_len) // self.page_tokens) - len(self.pages[slot]))
 
     def grow(self, slot: int, new_len: int) -> None:
         have = len(self.pages[slot])
-        want = -(-new_len // self.page_tokens)
+        want = -(-self.need.rows_of(new_len) // self.page_tokens)
         if want > self.max_pages_per_seq:
             raise CacheError(f"sequence of {new_len} tokens exceeds the cache's longest sequence "
                              f"({self.max_pages_per_seq * self.page_tokens})")

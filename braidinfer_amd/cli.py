@@ -90,7 +90,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     try:
         if args.random_weights is not None:
             import torch
-            cfg = B.preset(args.preset)
+            cfg = B.any_preset(args.preset)
             if args.save_folder:
                 where = args.save_folder
             else:

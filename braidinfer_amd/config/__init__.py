@@ -3,12 +3,26 @@ from .registry import (Architecture, register_architecture, unregister_architect
                        registered_architectures, architecture_of, architecture_of_config,
                        read_config_json, config_from_dict, config_from_folder, spec_of, generation_stop_tokens)
 from .mistral import MistralConfig, PRESETS, preset, build_spec as build_mistral_spec, ARCHITECTURE as MISTRAL
+from .kesitar import KesitarConfig, build_spec as build_kesitar_spec, ARCHITECTURE as KESITAR
+from . import kesitar as _kesitar
 
 register_architecture(MISTRAL, MistralConfig, build_mistral_spec, model_type="mistral", replace=True)
+register_architecture(KESITAR, KesitarConfig, build_kesitar_spec, model_type="kesitar", replace=True)
+PRESET_FAMILIES = {MISTRAL: (PRESETS, preset), KESITAR: (_kesitar.PRESETS, _kesitar.preset)}
+
+
+def any_preset(name: str, **overrides):
+    """A preset of any registered architecture by its name."""
+    for presets, make in PRESET_FAMILIES.values():
+        if name in presets:
+            return make(name, **overrides)
+    from ..errors import ConfigError
+    raise ConfigError(f"unknown preset {name!r}; known: {sorted(n for p, _ in PRESET_FAMILIES.values() for n in p)}")
 
 __all__ = [
     "PartSpec", "LayerSpec", "ScheduleEntry", "ModelSpec", "default_schedule", "prenorm_layer",
     "Architecture", "register_architecture", "unregister_architecture", "registered_architectures",
     "architecture_of", "architecture_of_config", "read_config_json", "config_from_dict",
     "config_from_folder", "spec_of", "generation_stop_tokens", "MistralConfig", "PRESETS", "preset",
+    "KesitarConfig", "any_preset", "PRESET_FAMILIES",
 ]

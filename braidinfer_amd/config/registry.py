@@ -2,8 +2,8 @@
 
 The reference has no registry: it sniffs keys (`layer_types`, `num_experts`, ...) and
 tests `model_type` strings (crates/braidinfer-runtime/src/config.rs:357-369,406-510).
-Here the key is ``config.json["architectures"][0]``, with `model_type` as a second
-name for folders that omit `architectures`.
+Here the key is ``config.json["architectures"][0]`` (or the one name under
+``"architecture"``), with `model_type` as a second name for folders that omit both.
 """
 from __future__ import annotations
 
@@ -48,7 +48,8 @@ def registered_architectures():
 
 
 def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
-    archs = config_dict.get("architectures")
+    # "architectures" (a list, as most checkpoints carry it) or "architecture" (one name)
+    archs = config_dict.get("architectures", config_dict.get("architecture"))
     name = None
     if isinstance(archs, (list, tuple)) and archs:
         name = archs[0]

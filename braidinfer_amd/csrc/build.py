@@ -36,6 +36,8 @@ MODULES: Dict[str, List[str]] = {
     "gemm_bf16": ["gemm_bf16.hip"],
     "attention_bf16": ["attention_bf16.hip"],
     "random_weights": ["random_weights.hip"],
+    "pooled_attention": ["pooled_attention.hip"],
+    "gated_recurrence": ["gated_recurrence.hip"],
 }
 HEADERS = ["common.h", "no_alloc.h"]
 

@@ -5,13 +5,13 @@
 #include "common.h"
 
 // ------------------------------------------------------------------ embedding ------
-// out[t, :] = float(table[token[t], :])            reference: op_embedding,
-// kernels/megakernel_ops.hip:1757-1768 (one instruction per token there; one launch
-// for all packed tokens here).  A token id outside the table writes zeros; the host
+// out[t, :] = float(table[token[t], :]) * scale    reference: op_embedding,
+// kernels/megakernel_ops.hip:1757-1768 (one instruction per token there, no scale; one
+// launch for all packed tokens here).  A token id outside the table writes zeros; the host
 // rejects such ids before the launch.
 template <typename W>
 __global__ void embedding_kernel(const W* __restrict__ table, const int* __restrict__ tokens,
-                                 float* __restrict__ out, int H, int V) {
+                                 float* __restrict__ out, int H, int V, float scale) {
     const int t = blockIdx.x;
     const int tok = tokens[t];
     float* o = out + (size_t)t * H;
@@ -20,18 +20,18 @@ __global__ void embedding_kernel(const W* __restrict__ table, const int* __restr
         return;
     }
     const W* r = table + (size_t)tok * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<W>(r[i]);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<W>(r[i]) * scale;
 }
 
 extern "C" int br_embedding(const void* table, int table_is_bf16, const int* tokens, float* out,
-                            int T, int H, int V, hipStream_t s) {
+                            int T, int H, int V, float scale, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (H <= 0 || V <= 0) return BR_BAD_ARG;
     int threads = H >= 1024 ? 256 : 64;
     if (table_is_bf16)
-        embedding_kernel<bf16><<<T, threads, 0, s>>>((const bf16*)table, tokens, out, H, V);
+        embedding_kernel<bf16><<<T, threads, 0, s>>>((const bf16*)table, tokens, out, H, V, scale);
     else
-        embedding_kernel<float><<<T, threads, 0, s>>>((const float*)table, tokens, out, H, V);
+        embedding_kernel<float><<<T, threads, 0, s>>>((const float*)table, tokens, out, H, V, scale);
     return br_check_launch();
 }
 
@@ -102,6 +102,60 @@ extern "C" int br_rmsnorm(const float* x, const float* w, void* y, int y_is_bf16
         if (y_is_bf16) rmsnorm_kernel<bf16><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps);
         else rmsnorm_kernel<float><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps);
     }
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------------ layer norm -----
+// y = (x - mean) / sqrt(var + eps) * w with var the mean of the squared deviations, no bias;
+// statistics in float, two passes over the row (the mean first, then the deviations), each
+// reduced by a fixed tree.  `center` 0 leaves the mean out: the RMS norm.  `rows` gathers as in
+// the RMS norm above.  With `add` the normed row is added to the float row `y` instead of
+// stored: y += norm(x) * w, the sum of a branch whose output is normed before it joins the
+// residual rows.
+template <typename T, bool ADD>
+__global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ y,
+                                 const int* __restrict__ rows, int H, float eps, int center) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * H;
+    T* yr = y + (size_t)r * H;
+    float mean = 0.f;
+    if (center) {
+        float sm = 0.f;
+        for (int i = threadIdx.x; i < H; i += blockDim.x) sm += xr[i];
+        mean = block_sum(sm, scratch) / (float)H;
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) { const float v = xr[i] - mean; ss += v * v; }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = (xr[i] - mean) * inv * w[i];
+        if (ADD) yr[i] = from_f32<T>(to_f32<T>(yr[i]) + v);
+        else yr[i] = from_f32<T>(v);
+    }
+}
+
+extern "C" int br_layernorm(const float* x, const float* w, void* y, int y_is_bf16, const int* rows, int R, int H,
+                            float eps, int center, int add, hipStream_t s) {
+    if (R <= 0) return BR_OK;
+    if (H <= 0 || (add && (y_is_bf16 || rows))) return BR_BAD_ARG;
+    const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
+    if (add) layernorm_kernel<float, true><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
+    else if (y_is_bf16) layernorm_kernel<bf16, false><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps, center);
+    else layernorm_kernel<float, false><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------------- row scale -----
+// x[i] *= scale (float), e.g. logits of a head with a fixed output scale.
+__global__ void scale_kernel(float* __restrict__ x, float scale, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] *= scale;
+}
+
+extern "C" int br_scale(float* x, float scale, size_t n, hipStream_t s) {
+    if (n == 0) return BR_OK;
+    scale_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, scale, n);
     return br_check_launch();
 }
 

@@ -98,9 +98,17 @@ class DecoderModel:
                 elif e.cache not in written:
                     raise ConfigError(f"schedule entry reads cache {e.cache} before any entry writes it")
         for e in self.schedule:
-            unknown = sorted(set(e.more_caches) - set(self.layers[e.layer].more_mixers))
+            layer = self.layers[e.layer]
+            own = set(layer.mixer.more_cache_needs()) if layer.mixer is not None else set()
+            both = sorted(own & set(layer.more_mixers))
+            if both:
+                raise ConfigError(f"layer {e.layer}: {both} name a further mixer and a further cache unit of the mixer")
+            unknown = sorted(set(e.more_caches) - set(layer.more_mixers) - own)
             if unknown:
                 raise ConfigError(f"schedule entry of layer {e.layer} names cache units for mixers the layer has not: {unknown}")
+            missing = sorted(own - set(e.more_caches)) if e.cache is not None else []
+            if missing:
+                raise ConfigError(f"schedule entry of layer {e.layer} names no cache units for its mixer's {missing}")
         for layer in self.layers:
             for m in self._mixers_of(layer).values():
                 m.check_positions(self.positions)
@@ -178,6 +186,14 @@ class DecoderModel:
                     raise ConfigError(f"cache unit {unit} is shared by mixers with different needs: "
                                       f"{needs[unit]} and {n}")
                 needs[unit] = n
+                # the mixer's further units (e.g. pooled rows) under the roles it names
+                for more_role, mn in (m.more_cache_needs().items() if role is None else ()):
+                    mu = e.more_caches.get(more_role)
+                    if mu is None:
+                        continue
+                    if mu in needs and needs[mu] != mn:
+                        raise ConfigError(f"cache unit {mu} is shared by mixers with different needs: {needs[mu]} and {mn}")
+                    needs[mu] = mn
         return needs
 
     def state_needs(self) -> Dict[object, StateNeed]:
@@ -239,6 +255,9 @@ class DecoderModel:
                    else MixerContext(unit=e.cache, writes_cache=e.writes_cache))
             for role in layer.more_mixers:
                 ctx.others[role] = self._mixer_context(cache, e, i, role)
+            if layer.mixer is not None:
+                for role in layer.mixer.more_cache_needs():
+                    ctx.others[role] = self._mixer_context(cache, e, i, role)
             layer.run(layer, x, step, ctx)
         if logits_out is None:
             logits = torch.empty((n_want, self.spec.vocab_size), dtype=torch.float32, device=rt.device)

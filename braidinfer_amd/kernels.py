@@ -83,14 +83,14 @@ def device_cus() -> int:
 
 
 # ------------------------------------------------------------------ elementwise -----
-def embedding(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+def embedding(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
     _dev("embedding", table, tokens, out)
     T = tokens.numel()
     V, H = table.shape
     _req(tokens.dtype == torch.int32, "embedding: tokens must be int32")
     _req(out.dtype == torch.float32 and out.shape == (T, H), "embedding: out must be float32 [T, H]")
-    f = _fn("elementwise", "br_embedding", [_P, c_int, _P, _P, c_int, c_int, c_int, _P])
-    _check(f(_ptr(table), _is_bf16(table, "embedding"), _ptr(tokens), _ptr(out), T, H, V, _stream()), "embedding")
+    f = _fn("elementwise", "br_embedding", [_P, c_int, _P, _P, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(table), _is_bf16(table, "embedding"), _ptr(tokens), _ptr(out), T, H, V, float(scale), _stream()), "embedding")
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,
@@ -107,6 +107,32 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,
     f = _fn("elementwise", "br_rmsnorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, _P])
     _check(f(_ptr(x), _ptr(w), _ptr(out), _is_bf16(out, "rmsnorm"), _ptr(rows), R, H, float(eps), _stream()),
            "rmsnorm")
+
+
+def layernorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
+              center: bool = True, add: bool = False) -> None:
+    """out = norm(x) * w, or out += norm(x) * w with `add` (float `out`); `center` False: the RMS norm."""
+    _dev("layernorm", x, w, out, rows)
+    H = x.shape[-1]
+    R = out.shape[0]
+    _req(x.dtype == torch.float32 and w.dtype == torch.float32, "layernorm: x and w must be float32")
+    _req(w.numel() == H and out.shape[-1] == H, "layernorm: widths of x, w and out differ")
+    if rows is None:
+        _req(x.shape[0] == R, "layernorm: out has other rows than x")
+    else:
+        _req(rows.dtype == torch.int32 and rows.numel() == R, "layernorm: rows must be int32 [R]")
+    _req(not add or (out.dtype == torch.float32 and rows is None and out.data_ptr() != x.data_ptr()),
+         "layernorm: adding needs float rows of their own, without a gather")
+    f = _fn("elementwise", "br_layernorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, c_int, c_int, _P])
+    _check(f(_ptr(x), _ptr(w), _ptr(out), _is_bf16(out, "layernorm"), _ptr(rows), R, H, float(eps), int(center),
+             int(add), _stream()), "layernorm")
+
+
+def scale_(x: torch.Tensor, scale: float) -> None:
+    _dev("scale", x)
+    _req(x.dtype == torch.float32, "scale: float32 only")
+    f = _fn("elementwise", "br_scale", [_P, c_float, c_size_t, _P])
+    _check(f(_ptr(x), float(scale), x.numel(), _stream()), "scale")
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
@@ -478,6 +504,125 @@ def attention_simple(q: torch.Tensor, q_stride: int, out: torch.Tensor, position
     _check(f(_ptr(q), q_stride, _ptr(out), _is_bf16(q, "attention_simple"), _ptr(positions), _ptr(seq_of_token),
              _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(cache), T, nq, nkv, hd, page,
              int(window or 0), float(scale), _stream()), "attention_simple")
+
+# -------------------------------------------- window attention with pooled blocks -----
+def _pwa_unit(name: str, unit: torch.Tensor, nkv: int, dk: int, dv: int, page: int) -> None:
+    _req(unit.dim() >= 2 and unit[0].numel() == nkv * page * (dk + dv),
+         f"{name}: a page of the cache unit must hold {nkv} heads x {page} rows x ({dk} + {dv})")
+
+
+def pwa_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm: Optional[torch.Tensor],
+                k_norm: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                rotary_dim: int, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
+                block_table: torch.Tensor, q_out: torch.Tensor, unit: torch.Tensor, v_first: Optional[torch.Tensor],
+                mix: Optional[torch.Tensor], v_role: int, nq: int, nkv: int, dk: int, dv: int, page: int,
+                write_cache: bool) -> None:
+    """Float projection sums [T, nq*dk + nkv*dk + nkv*dv] -> queries (normed, rotated) in `q_out` and the
+    tokens' keys (normed, rotated) and values in their cache pages.  `v_role` 1 leaves the values in
+    `v_first`, 2 mixes them with it by the scalar `mix`."""
+    _dev("pwa_prepare", qkv, bias, q_norm, k_norm, cos, sin, positions, seq_of_token, slots, block_table, q_out, unit,
+         v_first, mix)
+    T = qkv.shape[0]
+    width = nq * dk + nkv * dk + nkv * dv
+    _req(qkv.dtype == torch.float32 and qkv.shape == (T, width), "pwa_prepare: projections must be float32 [T, nq*dk + nkv*(dk+dv)]")
+    _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == width), "pwa_prepare: bias float32 of the projections' width")
+    for nw in (q_norm, k_norm):
+        _req(nw is None or (nw.dtype == torch.float32 and nw.numel() == dk), "pwa_prepare: norm weights float32 [dk]")
+    _req(positions.numel() >= T and seq_of_token.numel() >= T, "pwa_prepare: positions shorter than tokens")
+    _req(block_table.dim() == 2 and block_table.dtype == torch.int32, "pwa_prepare: block table int32 [slots, pages]")
+    _req(q_out.shape == (T, nq * dk) and q_out.dtype == unit.dtype, "pwa_prepare: q_out [T, nq*dk] of the cache's dtype")
+    _pwa_unit("pwa_prepare", unit, nkv, dk, dv, page)
+    if rotary_dim:
+        _req(cos is not None and sin is not None and cos.dtype == sin.dtype == torch.float32
+             and cos.numel() >= T * (rotary_dim // 2) and sin.numel() >= T * (rotary_dim // 2), "pwa_prepare: rotary tables float32 [T, rotary_dim/2]")
+    if v_role:
+        _req(v_first is not None and v_first.dtype == torch.float32 and v_first.numel() >= T * nkv * dv,
+             "pwa_prepare: v_first float32 [T, nkv*dv]")
+        _req(v_role != 2 or (mix is not None and mix.dtype == torch.float32 and mix.numel() == 1), "pwa_prepare: mix is one float")
+    f = _fn("pooled_attention", "br_pwa_prepare",
+            [_P, _P, _P, _P, c_float, _P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P, _P] + [c_int] * 8 + [_P])
+    _check(f(_ptr(qkv), _ptr(bias), _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(cos), _ptr(sin), int(rotary_dim),
+             _ptr(positions), _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1], _ptr(q_out),
+             _ptr(unit), _is_bf16(unit, "pwa_prepare"), _ptr(v_first), _ptr(mix), int(v_role), T, nq, nkv, dk, dv, page,
+             int(write_cache), _stream()), "pwa_prepare")
+
+
+def pwa_pool(unit: torch.Tensor, block_table: torch.Tensor, pooled: torch.Tensor, pooled_table: torch.Tensor,
+             cu_seqlens: torch.Tensor, ctx_lens: torch.Tensor, slots: torch.Tensor, B: int, max_new: int, nkv: int,
+             dk: int, dv: int, page: int, pool: int) -> None:
+    """Rows of the pooled unit for the blocks of `pool` tokens that this step completed: the means of
+    their keys and of their values as the token unit holds them."""
+    _dev("pwa_pool", unit, block_table, pooled, pooled_table, cu_seqlens, ctx_lens, slots)
+    _req(unit.dtype == pooled.dtype, "pwa_pool: both units share a dtype")
+    _pwa_unit("pwa_pool", unit, nkv, dk, dv, page)
+    _pwa_unit("pwa_pool", pooled, nkv, dk, dv, page)
+    _req(cu_seqlens.numel() >= B + 1 and ctx_lens.numel() >= B and slots.numel() >= B, "pwa_pool: arrays shorter than the batch")
+    for tb in (block_table, pooled_table):
+        _req(tb.dim() == 2 and tb.dtype == torch.int32, "pwa_pool: block tables int32 [slots, pages]")
+    f = _fn("pooled_attention", "br_pwa_pool", [_P, _P, c_int, _P, _P, c_int, _P, _P, _P] + [c_int] * 8 + [_P])
+    _check(f(_ptr(unit), _ptr(block_table), block_table.shape[1], _ptr(pooled), _ptr(pooled_table), pooled_table.shape[1],
+             _ptr(cu_seqlens), _ptr(ctx_lens), _ptr(slots), _is_bf16(unit, "pwa_pool"), B, max_new, nkv, dk, dv, page, pool,
+             _stream()), "pwa_pool")
+
+
+def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
+               block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
+               pooled: Optional[torch.Tensor], nq: int, nkv: int, dk: int, dv: int, page: int, size: int, pool: int,
+               scale: float, sink: bool) -> None:
+    """One wave per (query, head), float arithmetic: the window's tokens and the pooled blocks before it."""
+    _dev("pwa_attend", q, out, positions, seq_of_token, slots, block_table, unit, pooled_table, pooled)
+    T = q.shape[0]
+    _req(q.shape == (T, nq * dk) and out.shape == (T, nq * dv) and q.dtype == out.dtype == unit.dtype,
+         "pwa_attend: q [T, nq*dk], out [T, nq*dv], both of the cache's dtype")
+    _pwa_unit("pwa_attend", unit, nkv, dk, dv, page)
+    if pool:
+        _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_attend: pooled unit missing")
+        _pwa_unit("pwa_attend", pooled, nkv, dk, dv, page)
+    f = _fn("pooled_attention", "br_pwa_attend",
+            [_P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P])
+    _check(f(_ptr(q), _ptr(out), _is_bf16(q, "pwa_attend"), _ptr(positions), _ptr(seq_of_token), _ptr(slots),
+             _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
+             pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), T, nq, nkv, dk, dv, page, int(size),
+             int(pool), float(scale), int(sink), _stream()), "pwa_attend")
+
+
+# ------------------------------------------------------ gated linear recurrence -----
+def glr_gates(rows: torch.Tensor, f_bias: Optional[torch.Tensor], lower: Optional[torch.Tensor], hd: int) -> None:
+    """rows [T, 2*hd + .] float: the first hd columns become silu(.), the next hd the forget gate
+    lower + (1 - lower) * sigmoid(. + f_bias)."""
+    _dev("glr_gates", rows, f_bias, lower)
+    _req(rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape[1] >= 2 * hd, "glr_gates: rows float32 [T, >= 2*hd]")
+    for v in (f_bias, lower):
+        _req(v is None or (v.dtype == torch.float32 and v.numel() == hd), "glr_gates: bias and lower bound float32 [hd]")
+    f = _fn("gated_recurrence", "br_glr_gates", [_P, _P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(rows), _ptr(f_bias), _ptr(lower), rows.shape[0], hd, rows.shape[1], _stream()), "glr_gates")
+
+
+def glr_scan(rows: torch.Tensor, out: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor,
+             B: int, H: int, d: int, e: int) -> None:
+    """rows [T, 2*H*d + H*e] float (q | f | v, gates applied), state [slots, H, d, e] float: walks every
+    sequence's new tokens in order, writes o [T, H*e] float and leaves the state."""
+    _dev("glr_scan", rows, out, cu_seqlens, slots)
+    T = rows.shape[0]
+    _req(state.is_cuda and state.dim() == 4 and state[0].is_contiguous() and state.stride(0) >= H * d * e,
+         "glr_scan: every slot's state must be dense")
+    _req(rows.dtype == out.dtype == state.dtype == torch.float32, "glr_scan: float32 only")
+    _req(rows.shape == (T, 2 * H * d + H * e) and out.shape == (T, H * e), "glr_scan: rows [T, 2*H*d + H*e], out [T, H*e]")
+    _req(state.dim() == 4 and state.shape[1:] == (H, d, e), "glr_scan: state [slots, H, d, e]")
+    _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "glr_scan: arrays shorter than the batch")
+    _req(d <= 512, f"glr_scan: {d} query channels a head are beyond the kernel's 512")
+    f = _fn("gated_recurrence", "br_glr_scan", [_P, _P, _P, _P, _P] + [c_int] * 5 + [c_size_t, _P])
+    _check(f(_ptr(rows), _ptr(out), _ptr(state), _ptr(cu_seqlens), _ptr(slots), B, H, d, e, rows.shape[1],
+             state.stride(0), _stream()), "glr_scan")
+
+
+def head_rmsnorm(o: torch.Tensor, w: Optional[torch.Tensor], out: torch.Tensor, H: int, e: int, eps: float) -> None:
+    _dev("head_rmsnorm", o, w, out)
+    T = o.shape[0]
+    _req(o.dtype == torch.float32 and o.shape == (T, H * e) and out.shape == (T, H * e), "head_rmsnorm: o float32 [T, H*e]")
+    _req(w is None or (w.dtype == torch.float32 and w.numel() == e), "head_rmsnorm: weight float32 [e]")
+    f = _fn("gated_recurrence", "br_glr_head_norm", [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(o), _ptr(w), _ptr(out), _is_bf16(out, "head_rmsnorm"), T, H, e, float(eps), _stream()), "head_rmsnorm")
 
 
 def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu_seqlens: torch.Tensor,

@@ -87,6 +87,11 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def add_normed(self, y: torch.Tensor, x: torch.Tensor) -> None:
+        """x += norm(y), both float [T, H]: the sum of a branch whose output is normed before it
+        joins the residual rows.  Norms without a kernel for it norm into a buffer and add."""
+        raise NotImplementedError
+
     def prepare_in_product(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, ws) -> Any:
         """x += a @ w^T with this norm of the new x prepared in the same kernel, if the norm
         has such a kernel for these sizes and types: returns what `product_of_prepared`
@@ -123,8 +128,10 @@ class ResidualSink:
     next.  `linear(a, w, sink, ws, accumulate=True)` adds the product and, where the norm
     can, leaves its preparation in `prepared`."""
 
-    def __init__(self, x: torch.Tensor, next_norm: Optional["Norm"]):
-        self.x, self.next_norm, self.prepared = x, next_norm, None
+    def __init__(self, x: torch.Tensor, next_norm: Optional["Norm"], overwrite: bool = False):
+        # `overwrite`: the rows are a branch's own output, not the residual rows: a product "added" to
+        # them is stored (an arrangement that norms a branch's output before the sum hands such a sink)
+        self.x, self.next_norm, self.prepared, self.overwrite = x, next_norm, None, overwrite
 
 
 class NormedInput:
@@ -180,6 +187,12 @@ class Mixer(Part):
 
     def state_need(self) -> Optional[StateNeed]:
         return None
+
+    def more_cache_needs(self) -> Dict[str, CacheNeed]:
+        """Further cache units of this one mixer, by a role of its choosing (rows it keeps beside
+        its keys and values, e.g. one pooled row per block of tokens).  The run order names their
+        units in `ScheduleEntry.more_caches[role]`; the mixer finds them as `ctx.others[role]`."""
+        return {}
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, step, ctx: "MixerContext") -> None:
         """Add the mixer's output for the step's tokens to `x` in place."""

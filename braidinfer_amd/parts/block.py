@@ -57,4 +57,42 @@ class PrenormResidual:
             step.probe(f"L{step.schedule_index}.post_ffn", x)
 
 
+class SandwichResidual:
+    """x += norm_out(part(norm_in(x))) for the mixer and then for the feed-forward: a norm in front
+    of each half and one behind it, before the sum.  Roles of `layer.norms`: "mixer", "mixer_out",
+    "feed_forward", "feed_forward_out" (an absent one is left out).  The half writes its output
+    into float rows of its own; the norm behind it adds the normed rows to the residual rows, so
+    the sum is a float add in that kernel."""
+
+    def run(self, layer, x, step, mixer_ctx) -> None:
+        step.prepared_norm = None
+        if layer.mixer is not None:
+            self.branch(layer.mixer, layer.norms.get("mixer"), layer.norms.get("mixer_out"), x, step, layer.rt.dtype, mixer_ctx)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_mixer", x)
+        if layer.feed_forward is not None:
+            self.branch(layer.feed_forward, layer.norms.get("feed_forward"), layer.norms.get("feed_forward_out"), x, step,
+                        layer.rt.dtype)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_ffn", x)
+
+    @staticmethod
+    def branch(part, norm_in, norm_out, x, step, dtype, *extra) -> None:
+        h = x
+        if norm_in is not None:
+            h = step.ws.get("block_h", tuple(x.shape), dtype)
+            norm_in.forward(x, h)
+        if norm_out is None:
+            part.forward(h, x, step, *extra)
+            return
+        y = step.ws.get("branch_out", tuple(x.shape), x.dtype)
+        if part.through_linear_only:
+            part.forward(h, ResidualSink(y, None, overwrite=True), step, *extra)
+        else:
+            y.zero_()
+            part.forward(h, y, step, *extra)
+        norm_out.add_normed(y, x)
+
+
 register_part("block", "prenorm_residual", PrenormResidual, replace=True)
+register_part("block", "sandwich_residual", SandwichResidual, replace=True)

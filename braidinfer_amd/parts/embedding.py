@@ -1,9 +1,10 @@
 """Token embedding and output head.
 
-x[t] = float(embed[token[t]]), no scaling (reference: op_embedding,
-kernels/megakernel_ops.hip:1757-1768); logits = W_lm n in float, no bias, no soft cap
-(op_lm_head, :1783-1835); a tied head uses the embedding tensor itself
-(model_load.rs:388-398)."""
+x[t] = float(embed[token[t]]) * scale, scale 1 by default (reference: op_embedding,
+kernels/megakernel_ops.hip:1757-1768, which has no scale); logits = W_lm n * scale in float, no
+bias, no soft cap (op_lm_head, :1783-1835, no scale either); a tied head uses the embedding
+tensor itself, without the embedding's scale (model_load.rs:388-398).  `tensor` is the piece of
+the table's name behind the part's prefix."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -20,27 +21,27 @@ from .linear import linear, stream_layout
 class TokenEmbedding(Embedding):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
-        self.V, self.H = int(vocab_size), int(hidden_size)
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensor: str = "weight"):
+        self.V, self.H, self.scale, self.tensor = int(vocab_size), int(hidden_size), float(scale), tensor
         self.weight = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(prefix + "weight", (self.V, self.H))]
+        return [TensorSpec(prefix + self.tensor, (self.V, self.H))]
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = rt.own(tensors[prefix + "weight"])
-        rt.published[prefix + "weight"] = self.weight      # a tied output head reads the same table
+        self.weight = rt.own(tensors[prefix + self.tensor])
+        rt.published[prefix + self.tensor] = self.weight      # a tied output head reads the same table
 
     def forward(self, tokens, out) -> None:
-        K.embedding(self.weight, tokens, out)
+        K.embedding(self.weight, tokens, out, self.scale)
 
 
 class LMHead(OutputHead):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None):
-        self.V, self.H, self.tied_to = int(vocab_size), int(hidden_size), tied_to
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, scale: float = 1.0):
+        self.V, self.H, self.tied_to, self.scale = int(vocab_size), int(hidden_size), tied_to, float(scale)
         self.weight = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
@@ -67,6 +68,8 @@ class LMHead(OutputHead):
 
     def forward(self, h, out, ws=None) -> None:
         linear(h, self.weight, out, ws)
+        if self.scale != 1.0:
+            K.scale_(out, self.scale)
 
 
 register_part("embedding", "embedding", TokenEmbedding, replace=True)

@@ -3,7 +3,7 @@
 :1559-1602; the activation is fixed to SiLU there, :1538-1544)."""
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -17,25 +17,30 @@ class SwiGLU(FeedForward):
     graph_safe = True
     through_linear_only = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    def __init__(self, hidden_size: int, intermediate_size: int, names: Optional[Dict[str, str]] = None):
+        """`names`: the pieces of the three matrices' names behind the part's prefix, for checkpoints
+        that call them otherwise than "gate_proj.weight", "up_proj.weight", "down_proj.weight"."""
         self.H, self.I = int(hidden_size), int(intermediate_size)
+        self.names = dict(self.NAMES, **(names or {}))
         self.w_gu = self.w_d = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
         return [
-            TensorSpec(prefix + "gate_proj.weight", (self.I, self.H)),
-            TensorSpec(prefix + "up_proj.weight", (self.I, self.H)),
-            TensorSpec(prefix + "down_proj.weight", (self.H, self.I)),
+            TensorSpec(prefix + self.names["gate"], (self.I, self.H)),
+            TensorSpec(prefix + self.names["up"], (self.I, self.H)),
+            TensorSpec(prefix + self.names["down"], (self.H, self.I)),
         ]
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        g, u = tensors[prefix + "gate_proj.weight"], tensors[prefix + "up_proj.weight"]
+        g, u = tensors[prefix + self.names["gate"]], tensors[prefix + self.names["up"]]
         # bf16: gate and up rows interleaved so that the product's epilogue applies silu * up
         # and the [T, 2 I] intermediate is never written
         self.fused = g.dtype == u.dtype == torch.bfloat16 and rt.is_bf16 and self.I % 8 == 0
         self.w_gu = fused_layout([g, u], rt, interleave=self.fused)
-        self.w_d = stream_layout(tensors[prefix + "down_proj.weight"], rt)
+        self.w_d = stream_layout(tensors[prefix + self.names["down"]], rt)
 
     def forward(self, h, x, step) -> None:
         T = step.n_tokens

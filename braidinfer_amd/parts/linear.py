@@ -27,6 +27,8 @@ def linear(a, w: torch.Tensor, out, ws, accumulate: bool = False) -> None:
         a = a.tensor()
     if isinstance(out, ResidualSink):
         sink, out = out, out.x
+        if sink.overwrite:
+            accumulate = False
         if accumulate and sink.next_norm is not None:
             sink.prepared = sink.next_norm.prepare_in_product(a, w, out, ws)
             if sink.prepared is not None:

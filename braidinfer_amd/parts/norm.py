@@ -1,5 +1,11 @@
 """RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, plain `w` (reference: op_rmsnorm_wx,
-kernels/megakernel_ops.hip:862-904; eps default and key in config.rs:249-252)."""
+kernels/megakernel_ops.hip:862-904; eps default and key in config.rs:249-252).
+
+LayerNorm: y = (x - mean) / sqrt(var + eps) * w, var the mean of the squared deviations, a weight
+and no bias (absent in the reference, whose models norm without centering).
+
+`tensor` is the piece of the weight's name behind the part's prefix ("weight" in the
+checkpoints the reference loads; "" where the prefix is the whole name)."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -14,20 +20,23 @@ from .base import Norm, ProductRuns, Runtime, register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = int(size), float(eps)
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+        self.size, self.eps, self.tensor = int(size), float(eps), tensor
         self.weight: Optional[torch.Tensor] = None
 
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(prefix + "weight", (self.size,), kind="vector", init="ones")]
+        return [TensorSpec(prefix + self.tensor, (self.size,), kind="vector", init="ones")]
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        self.weight = rt.own(tensors[prefix + "weight"].to(torch.float32))
+        self.weight = rt.own(tensors[prefix + self.tensor].to(torch.float32))
 
     def forward(self, x, out, rows=None):
         K.rmsnorm(x, self.weight, out, self.eps, rows)
         return out
+
+    def add_normed(self, y, x):
+        K.layernorm(y, self.weight, x, self.eps, center=False, add=True)
 
     def prepare_in_product(self, a, w, x, ws):
         M, N = x.shape
@@ -59,4 +68,29 @@ class RMSNorm(Norm):
         return ProductRuns(scratch, runs, xg.shape[0], n_out) if runs else None
 
 
+class LayerNorm(Norm):
+    """Centered norm with a weight and no bias; statistics in float in both precisions."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+        self.size, self.eps, self.tensor = int(size), float(eps), tensor
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        return [TensorSpec(prefix + self.tensor, (self.size,), kind="vector", init="ones")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        self.weight = rt.own(tensors[prefix + self.tensor].to(torch.float32))
+
+    def forward(self, x, out, rows=None):
+        K.layernorm(x, self.weight, out, self.eps, rows, center=True)
+        return out
+
+    def add_normed(self, y, x):
+        K.layernorm(y, self.weight, x, self.eps, center=True, add=True)
+
+
 register_part("norm", "rmsnorm", RMSNorm, replace=True)
+register_part("norm", "layernorm", LayerNorm, replace=True)

@@ -1,0 +1,186 @@
+"""Grouped-query attention over a sliding window and pooled blocks of what left it.
+
+Per token: q, k, v = W n (+ bias); q and k are RMS-normed per head (one weight of the head's
+width, shared by the heads) and rotated on the first `rotary_dim` elements by the position
+encoding the mixer names; the values may be mixed with the values another layer made of the
+same token, v <- (1 - m) v + m v_first with a learnt scalar m.  Keys (normed, rotated) and
+values (mixed) are what the cache keeps.  A query at position i sees the tokens j with
+0 <= i - j < window and, for every block b of `pool` tokens with b pool + pool - 1 <= i - window,
+one pooled key and value: the means of the block's keys and of its values as the cache holds
+them.  Tokens that left the window and whose block is not complete behind it are not seen.
+Tokens and blocks share one softmax of the scores (q . k) * scale, which may carry a sink: a key
+of score 0 without a value, i.e. one added to the denominator.  Key and value widths may differ.
+
+Cache: the mixer's own unit keeps the tokens' rows as long as a later query or a block that is
+not pooled yet needs them (`CacheNeed.live_from`); a further unit under the role "pooled" keeps
+one row per block (`CacheNeed.tokens_per_row`).  Scores, softmax weights, norms and angles are
+float in both precisions.  Nothing of this is in the reference, whose attention is full and
+causal (kernels/megakernel_ops.hip:2150-2343).
+"""
+from __future__ import annotations
+
+import functools
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import kernels as K
+from ..cache import CacheNeed
+from ..errors import ConfigError, StepError
+from ..weights import TensorSpec
+from .base import Mixer, MixerContext, RotaryTables, Runtime, register_part
+from .linear import fused_layout, linear, stream_layout
+
+MAX_WIDTH = 512      # of a head's keys or values: the kernels' limit
+
+
+@functools.lru_cache(maxsize=None)
+def window_and_open_block(window: int, pool: int):
+    """`CacheNeed.live_from` of a window with pooled blocks: at length L the next query sees tokens
+    from L - window + 1 on, and the block that is still open (from pool * floor(L / pool) on) has yet to be
+    pooled.  One function object per (window, pool), so that layers with equal sizes share a group."""
+    def first_live(length: int) -> int:
+        first = length - window + 1
+        if pool > 0:
+            first = min(first, (length // pool) * pool)
+        return max(0, first)
+    return first_live
+
+
+class PooledWindowAttention(Mixer):
+    graph_safe = True
+    through_linear_only = True
+
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
+                 window: int, pool: int = 0, scale: Optional[float] = None, sink: bool = False, bias: bool = False,
+                 qk_norm_eps: Optional[float] = None, position: Optional[str] = None,
+                 value_mix: Optional[str] = None, value_mix_group: str = "v_first",
+                 names: Optional[Dict[str, str]] = None):
+        """`qk_norm_eps` None: no query/key norm.  `value_mix`: None, "source" (this layer's values are what
+        later layers of the same `value_mix_group` mix with; its own scalar is loaded and unused) or "mix"."""
+        if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+            raise ConfigError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if not 0 < key_dim <= MAX_WIDTH or not 0 < value_dim <= MAX_WIDTH:
+            raise ConfigError(f"attention: head widths {key_dim} (keys) and {value_dim} (values) must lie in 1..{MAX_WIDTH}")
+        if window is None or int(window) <= 0 or int(pool or 0) < 0:
+            raise ConfigError(f"attention: the window must be positive and the pooled block's size not negative, got {window}, {pool}")
+        if value_mix not in (None, "source", "mix"):
+            raise ConfigError(f"attention: value_mix must be None, 'source' or 'mix', got {value_mix!r}")
+        self.H, self.nq, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dk, self.dv = int(key_dim), int(value_dim)
+        self.window, self.pool = int(window), int(pool or 0)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
+        self.sink, self.bias = bool(sink), bool(bias)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.position = position
+        self.value_mix, self.value_mix_group = value_mix, value_mix_group
+        self.names = dict(self.NAMES, **(names or {}))
+        self.w_qkv = self.w_o = self.b_qkv = self.q_norm = self.k_norm = self.mix = None
+        self._expects_tables = False
+
+    # ---- weights -----------------------------------------------------------------------
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        n = self.names
+        out = [TensorSpec(prefix + n["q"], (self.nq * self.dk, self.H))]
+        if self.bias:
+            out.append(TensorSpec(prefix + n["q_bias"], (self.nq * self.dk,), kind="vector", init="normal"))
+        out.append(TensorSpec(prefix + n["k"], (self.nkv * self.dk, self.H)))
+        if self.bias:
+            out.append(TensorSpec(prefix + n["k_bias"], (self.nkv * self.dk,), kind="vector", init="normal"))
+        out.append(TensorSpec(prefix + n["v"], (self.nkv * self.dv, self.H)))
+        if self.bias:
+            out.append(TensorSpec(prefix + n["v_bias"], (self.nkv * self.dv,), kind="vector", init="normal"))
+        if self.qk_norm_eps is not None:
+            out += [TensorSpec(prefix + n["q_norm"], (self.dk,), kind="vector", init="ones"),
+                    TensorSpec(prefix + n["k_norm"], (self.dk,), kind="vector", init="ones")]
+        if self.value_mix is not None:
+            out.append(TensorSpec(prefix + n["value_mix"], (), kind="vector", init="normal"))
+        out.append(TensorSpec(prefix + n["o"], (self.H, self.nq * self.dv)))
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        self.w_qkv = fused_layout([tensors[prefix + n[x]] for x in ("q", "k", "v")], rt)
+        self.w_o = stream_layout(tensors[prefix + n["o"]], rt)
+        if self.bias:
+            self.b_qkv = rt.own(torch.cat([tensors[prefix + n[x]].to(torch.float32).reshape(-1) for x in ("q_bias", "k_bias", "v_bias")]))
+        if self.qk_norm_eps is not None:
+            self.q_norm = rt.own(tensors[prefix + n["q_norm"]].to(torch.float32))
+            self.k_norm = rt.own(tensors[prefix + n["k_norm"]].to(torch.float32))
+        if self.value_mix == "mix":
+            self.mix = rt.own(tensors[prefix + n["value_mix"]].to(torch.float32).reshape(1))
+
+    # ---- what it keeps -----------------------------------------------------------------
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(kv_heads=self.nkv, head_dim=self.dk, value_dim=self.dv,
+                         live_from=window_and_open_block(self.window, self.pool))
+
+    def more_cache_needs(self) -> Dict[str, CacheNeed]:
+        if not self.pool:
+            return {}
+        return {"pooled": CacheNeed(kv_heads=self.nkv, head_dim=self.dk, value_dim=self.dv, tokens_per_row=self.pool)}
+
+    def check_positions(self, encodings) -> None:
+        if self.position is None:
+            return
+        enc = encodings.get(self.position)
+        if enc is None:
+            raise ConfigError(f"attention asks for the position encoding {self.position!r}, the model has {sorted(encodings)}")
+        if getattr(enc, "gives", None) not in ("rotary", "embedding", "none"):
+            raise ConfigError(f"attention cannot use the position encoding {self.position!r}: it gives {getattr(enc, 'gives', None)!r}")
+        self._expects_tables = enc.gives == "rotary"
+        if self._expects_tables and (enc.rotary_dim > self.dk or getattr(enc, "pairing", "half") != "half"):
+            raise ConfigError(f"attention: the encoding {self.position!r} rotates {enc.rotary_dim} elements in "
+                              f"{getattr(enc, 'pairing', None)!r} pairs; this mixer takes up to {self.dk} in 'half' pairs")
+
+    # ---- one step ----------------------------------------------------------------------
+    def forward(self, h, x, step, ctx: MixerContext) -> None:
+        T = step.n_tokens
+        nq, nkv, dk, dv = self.nq, self.nkv, self.dk, self.dv
+        dt = self.rt.dtype
+        tables = step.position_data.get(self.position) if self.position else None
+        if (tables is None and self._expects_tables) or (tables is not None and not isinstance(tables, RotaryTables)):
+            raise StepError(f"attention: the position encoding {self.position!r} gave {type(tables).__name__}, "
+                            "rotary tables were expected")
+        if ctx.storage is None or (self.pool and "pooled" not in ctx.others):
+            raise StepError("attention: the run order gave this mixer no cache unit (or none for its pooled rows)")
+        # the projections' float sums: norms and angles work on them before anything is rounded
+        qkv = step.ws.get("pwa_qkv", (T, nq * dk + nkv * (dk + dv)), torch.float32)
+        linear(h, self.w_qkv, qkv, step.ws)
+        q = step.ws.get("pwa_q", (T, nq * dk), dt)
+        v_first, role = None, 0
+        if self.value_mix is not None:
+            key = ("value_mix", self.value_mix_group)
+            if self.value_mix == "source":
+                v_first = step.ws.get(f"pwa_{self.value_mix_group}", (T, nkv * dv), torch.float32)
+                step.extras[key] = v_first
+                role = 1
+            else:
+                v_first = step.extras.get(key)
+                if v_first is None or v_first.shape != (T, nkv * dv):
+                    raise StepError(f"attention: no layer before this one left values of width {nkv * dv} to mix with "
+                                    f"(group {self.value_mix_group!r})")
+                role = 2
+        unit = ctx.storage
+        K.pwa_prepare(qkv, self.b_qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0,
+                      tables.cos if tables else None, tables.sin if tables else None, tables.rotary_dim if tables else 0,
+                      step.positions, step.seq_of_token, step.slots, ctx.block_table, q, unit, v_first, self.mix, role,
+                      nq, nkv, dk, dv, ctx.page_tokens, ctx.writes_cache)
+        pooled = ctx.others.get("pooled")
+        if pooled is not None and ctx.writes_cache:
+            K.pwa_pool(unit, ctx.block_table, pooled.storage, pooled.block_table, step.cu_seqlens, step.ctx_lens, step.slots,
+                       step.n_seqs, step.max_new, nkv, dk, dv, ctx.page_tokens, self.pool)
+        o = step.ws.get("pwa_out", (T, nq * dv), dt)
+        K.pwa_attend(q, o, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit,
+                     pooled.block_table if pooled is not None else None, pooled.storage if pooled is not None else None,
+                     nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
+        linear(o, self.w_o, x, step.ws, accumulate=True)
+
+
+register_part("mixer", "pooled_window_attention", PooledWindowAttention, replace=True)
