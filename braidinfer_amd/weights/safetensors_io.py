@@ -189,7 +189,7 @@ class SafetensorsWriter:
                               f"got {name} {t.dtype} {list(t.shape)}")
         t = t.detach().cpu().contiguous()
         if n:
-            self._f.write(memoryview(t.view(torch.uint8).reshape(-1).numpy()))
+            self._f.write(memoryview(t.reshape(-1).view(torch.uint8).numpy()))      # reshape first: a scalar has no last dimension to split
         self._next += 1
 
     def close(self) -> None:

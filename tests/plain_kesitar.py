@@ -102,7 +102,8 @@ def attention_mixer(h, w, p, m, eps, v_first):
     """h [T, width]; `p` the layer's tensor prefix, `m` its mixer's sizes.  Returns the mixer's
     output and the values that were cached (what a later value-mixing layer takes as v_first)."""
     T = h.shape[0]
-    H, G, d, e = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, d, e = m["heads"], m["dim"], m["vdim"]
+    G = m.get("kv_heads", H)
     q = (h @ w[p + "q"].T + w[p + "q.b"]).reshape(T, H, d)
     k = (h @ w[p + "k"].T + w[p + "k.b"]).reshape(T, G, d)
     v = (h @ w[p + "v"].T + w[p + "v.b"]).reshape(T, G, e)
@@ -116,7 +117,8 @@ def attention_mixer(h, w, p, m, eps, v_first):
     if m.get("v_mix") and v_first is not None:
         lam = float(w[p + "vmix"])
         v = (1.0 - lam) * v + lam * v_first
-    o = pooled_window_attention(q, k, v, m["scale"], m["mask"]["size"], m["mask"]["pool"])
+    scale = m["scale"] if m.get("scale") is not None else d ** -0.5
+    o = pooled_window_attention(q, k, v, scale, m["mask"]["size"], m["mask"].get("pool") or 0)
     return o.reshape(T, H * e) @ w[p + "o"].T, v
 
 
@@ -195,3 +197,66 @@ def read_folder(folder):
             raise ValueError(f"{name}: dtype {t['dtype']}")
         w[name] = arr.reshape(t["shape"])
     return cfg, w
+
+
+def to_bf16(a):
+    """Round float values to the nearest bfloat16 (ties to even), returned as float64."""
+    u = np.asarray(a, dtype=np.float32).view(np.uint32)
+    r = ((u + (((u >> 16) & 1) + 0x7FFF)) >> 16).astype(np.uint32) << 16
+    return r.view(np.float32).astype(np.float64)
+
+
+def write_folder(folder, cfg, w):
+    """config.json and model.safetensors (bfloat16) of a configuration dict and float tensors."""
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    head, blobs, off = {}, [], 0
+    for name, a in w.items():
+        a32 = np.asarray(a, dtype=np.float32)
+        u = np.ascontiguousarray(a32).reshape(-1).view(np.uint32)
+        raw = ((u + (((u >> 16) & 1) + 0x7FFF)) >> 16).astype("<u2").tobytes()
+        head[name] = {"dtype": "BF16", "shape": list(a32.shape), "data_offsets": [off, off + len(raw)]}
+        off += len(raw)
+        blobs.append(raw)
+    hj = json.dumps(head).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(folder, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(hj)) + hj + b"".join(blobs))
+
+
+def random_weights(cfg, seed, gain=1.0):
+    """Random tensors (bfloat16 values) for a configuration dict: matrices N(0, gain^2 / fan-in), norm
+    weights around 1, biases N(0, 0.3^2), lower bounds in (0.05, 0.9), value mixing in (0.2, 0.8)."""
+    rng = np.random.default_rng(seed)
+    W, w = cfg["width"], {}
+
+    def mat(o, i):
+        return to_bf16(rng.standard_normal((o, i)) * gain / math.sqrt(i))
+
+    def vec(n, around=1.0, spread=0.3):
+        return to_bf16(around + spread * rng.standard_normal(n))
+    w["embed"] = to_bf16(rng.standard_normal((cfg["vocab"], W)))
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        for n in ["norm1", "norm1b"] + (["norm2", "norm2b"] if l.get("mlp") else []):
+            w[p + n] = vec(W)
+        H, d, e = m["heads"], m["dim"], m["vdim"]
+        if l["type"] == "attention":
+            G = m.get("kv_heads", H)
+            w[p + "mix.q"], w[p + "mix.q.b"] = mat(H * d, W), vec(H * d, 0.0)
+            w[p + "mix.k"], w[p + "mix.k.b"] = mat(G * d, W), vec(G * d, 0.0)
+            w[p + "mix.v"], w[p + "mix.v.b"] = mat(G * e, W), vec(G * e, 0.0)
+            w[p + "mix.q.norm"], w[p + "mix.k.norm"] = vec(d, 1.5), vec(d, 1.5)
+            if m.get("v_mix"):
+                w[p + "mix.vmix"] = to_bf16(rng.uniform(0.2, 0.8, ()))
+            w[p + "mix.o"] = mat(W, H * e)
+        else:
+            w[p + "mix.q"], w[p + "mix.f"], w[p + "mix.f.b"] = mat(H * d, W), mat(H * d, W), vec(H * d, 0.0, 1.0)
+            w[p + "mix.lower"] = to_bf16(rng.uniform(0.05, 0.9, H * d))
+            w[p + "mix.v"], w[p + "mix.norm"], w[p + "mix.o"] = mat(H * e, W), vec(e), mat(W, H * e)
+        if l.get("mlp"):
+            F = l["mlp"]["ff"]
+            w[p + "mlp.gate"], w[p + "mlp.up"], w[p + "mlp.down"] = mat(F, W), mat(F, W), mat(W, F)
+    w["final.norm"] = vec(W)
+    return w
