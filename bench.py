@@ -69,6 +69,12 @@ def measured_peaks(torch, K):
     return out
 
 
+LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_kv_write", "silu_mul", "residual_add", "gather_rows",
+             "convert", "gemm", "gemm_swiglu", "gemm_norm_prepare", "gemm_norm_scaled", "attention_simple",
+             "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16",
+             "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax"]
+
+
 def kernel_share(torch, eng, entries_of, classes):
     """Where the kernel time of one decode step goes: the step is run eagerly (no graph) with
     every launcher of `braidinfer_amd.kernels` bracketed by events; shares by class of kernel."""
@@ -85,9 +91,7 @@ def kernel_share(torch, eng, entries_of, classes):
             records.append((classes(name, a, k), s, e))
             return r
         return g
-    names = ["embedding", "rmsnorm", "rope_table", "rope_kv_write", "silu_mul", "residual_add", "gather_rows", "convert",
-             "gemm", "gemm_swiglu", "gemm_norm_prepare", "gemm_norm_scaled", "attention_simple",
-             "attention_prefill_bf16", "attention_decode_bf16", "argmax"]
+    names = LAUNCHERS
     was = eng.use_graphs
     eng.use_graphs = False
     try:
@@ -250,6 +254,160 @@ class Shape:
         return dt, self.weight_bytes + mean_ctx_total * self.kv_bytes_per_token, float(np.mean(lens)), shares
 
 
+# ------------------------------------------------- a design beside its closest model -----
+# `--design kesitar`: prompt and single-token throughput of the Kesitar design at the sizes of a real model's
+# layers, beside Mistral (the library's closest model: grouped-query attention, gated feed-forward) with the same
+# width, heads, feed-forward and number of layers, and the time of every kernel launcher in one prompt and one
+# single-token step of each (run eagerly, bracketed by events).
+DESIGN_SIZES = {
+    "kesitar": {
+        "1b": ("kesitar-1b", dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
+                                  intermediate_size=5632, vocab_size=32768, rope_theta=10000.0, rms_norm_eps=1e-6,
+                                  sliding_window=None, max_position_embeddings=32768)),
+        "7b": ("kesitar-7b", dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                                  intermediate_size=14336, vocab_size=32768, rope_theta=10000.0, rms_norm_eps=1e-6,
+                                  sliding_window=None, max_position_embeddings=32768)),
+    },
+}
+
+
+def launcher_times(torch, eng, run, reps=3):
+    """ms and calls by launcher of `braidinfer_amd.kernels` for what `run()` launches, eagerly (the last of `reps` runs)."""
+    from braidinfer_amd import kernels as K
+    records, saved = [], {}
+
+    def wrap(name, f):
+        def g(*a, **k):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            r = f(*a, **k)
+            e.record()
+            records.append((name, s, e))
+            return r
+        return g
+    was = eng.use_graphs
+    eng.use_graphs = False
+    try:
+        for n in LAUNCHERS:
+            saved[n] = getattr(K, n)
+            setattr(K, n, wrap(n, saved[n]))
+        for rep in range(reps):
+            records.clear()
+            run()
+            torch.cuda.synchronize()
+    finally:
+        for n, f in saved.items():
+            setattr(K, n, f)
+        eng.use_graphs = was
+    out = {}
+    for name, s, e in records:
+        ms, calls = out.get(name, (0.0, 0))
+        out[name] = (ms + s.elapsed_time(e), calls + 1)
+    return {k: {"ms": round(v[0], 4), "calls": v[1]} for k, v in sorted(out.items(), key=lambda kv: -kv[1][0])}
+
+
+def measure_design(torch, B, name, config, vocab, prompts, batches, context, steps, warmup):
+    from braidinfer_amd import StepEntry
+    from braidinfer_amd.sampling import Sampler
+    room = max(max(prompts), max(batches) * (context + 64)) + 4096
+    t0 = time.time()
+    eng = B.Engine.random(config, seed=0, dtype="bfloat16", max_tokens=room, max_seq_len=max(max(prompts), context + steps + warmup + 8))
+    print(f"[bench] {name}: engine ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    sampler = Sampler(eng.device, vocab)
+    rng = np.random.default_rng(7)
+    out = {"prefill": {}, "decode": {}, "kernels": {}}
+    for T in prompts:
+        prompt = [int(t) for t in rng.integers(0, vocab, T)]
+        times = []
+        for rep in range(4):
+            s = eng.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([StepEntry(s, prompt, [T - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.free_slot(s)
+        out["prefill"][str(T)] = {"tokens_per_s": round(T / min(times[1:]), 1), "ms": round(min(times[1:]) * 1e3, 3)}
+        print(f"[bench] {name}: prefill of {T}: {min(times[1:]) * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    for batch in batches:
+        ps = [[int(t) for t in rng.integers(0, vocab, context)] for _ in range(batch)]
+        slots = [eng.alloc_slot() for _ in range(batch)]
+        last = []
+        for i in range(0, batch, 8):
+            lg = eng.step([StepEntry(slots[b], ps[b], [context - 1]) for b in range(i, min(batch, i + 8))])
+            last.append(lg.clone())
+        toks = sampler.argmax(torch.cat(last)).tolist()
+        chain = eng.chain(slots, toks, None)
+
+        def one():
+            nonlocal toks
+            if chain is None:
+                toks = sampler.argmax(eng.step([StepEntry(slots[b], [toks[b]], [0]) for b in range(batch)])).tolist()
+            else:
+                chain.launch()
+                toks = chain.read()
+        if chain is not None:
+            chain.launch()
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t) / steps
+        if chain is not None:
+            chain.read()
+            chain.close()
+        for sl in slots:
+            eng.free_slot(sl)
+        out["decode"][str(batch)] = {"tokens_per_s": round(batch / dt, 1), "ms_per_step": round(dt * 1e3, 4)}
+        print(f"[bench] {name}: batch {batch}: {dt * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    for T in prompts:
+        prompt = [int(t) for t in rng.integers(0, vocab, T)]
+
+        def whole():
+            sl = eng.alloc_slot()
+            eng.step([StepEntry(sl, prompt, [T - 1])])
+            eng.free_slot(sl)
+        out["kernels"][f"prefill_{T}"] = launcher_times(torch, eng, whole)
+    # one single-token step of 8 sequences that hold `context` tokens each
+    slots = [eng.alloc_slot() for _ in range(8)]
+    ps = [[int(t) for t in rng.integers(0, vocab, context)] for _ in range(8)]
+    eng.step([StepEntry(slots[b], ps[b], []) for b in range(8)])
+    out["kernels"][f"decode_b8_ctx{context}"] = launcher_times(
+        torch, eng, lambda: eng.step([StepEntry(slots[b], [1], [0]) for b in range(8)]))
+    for sl in slots:
+        eng.free_slot(sl)
+    del eng, sampler
+    torch.cuda.empty_cache()
+    return out
+
+
+def design_comparison(args) -> int:
+    import torch
+    import braidinfer_amd as B
+    sizes = DESIGN_SIZES[args.design]
+    line = {"metric": f"{args.design} beside mistral at equal size: prefill and decode tokens/s, bf16, random weights",
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "layers": args.layers or 8,
+            "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+    prompts = [2048, 8192]
+    for size in (args.design_size.split(",") if args.design_size else sorted(sizes)):
+        preset_name, like = sizes[size]
+        L = args.layers or 8
+        full = B.any_preset(preset_name)
+        cfg = B.any_preset(preset_name, layers=[dict(l) for l in full.layers[:L]])
+        mistral = B.MistralConfig.from_dict(dict(like, num_hidden_layers=L))
+        got = {}
+        got[args.design] = measure_design(torch, B, f"{preset_name} ({L} layers)", cfg, cfg.vocab, prompts, [8, 64], 1024,
+                                          args.steps, args.warmup)
+        got["mistral"] = measure_design(torch, B, f"mistral of that size ({L} layers)", mistral, mistral.vocab_size, prompts,
+                                        [8, 64], 1024, args.steps, args.warmup)
+        line["sizes"][size] = got
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def room_for(batches, prompt_max, context, untimed_and_timed, prefill_tokens):
     per_seq = -(-(min(prompt_max, context) + untimed_and_timed + 3) // 64) * 64
     return max(max(batches) * per_seq, -(-prefill_tokens // 64) * 64)
@@ -274,12 +432,17 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true",
                     help="skip the further batch sizes, prompt lengths and workloads, the measured peaks and the kernel shares")
+    ap.add_argument("--design", default=None, choices=sorted(DESIGN_SIZES),
+                    help="instead of the workload: this design beside Mistral at equal size (prefill, decode, kernel times)")
+    ap.add_argument("--design-size", default=None, help="sizes of --design to run, with commas (default: all)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the prefill of --prefill-tokens (for profiles); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        return design_comparison(args)
     wl = WORKLOADS[args.workload]
     for k, v in wl.items():
         if getattr(args, k) is None:

@@ -135,14 +135,104 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
     }
 }
 
+// The same for widths in steps of 4 up to 4 * VPT * blockDim: a row is read once, 16 bytes a load, and kept
+// in registers between the sums and the scaling.  With `w2` the kernel goes on: the row it has just added
+// to (the residual row) is normed once more with the weight `w2` into `y2` (compute dtype): the norm
+// behind one half of a layer and the norm in front of the next in one pass over the row.
+template <typename T, typename T2, bool ADD, int VPT>
+__global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ y,
+                                     const int* __restrict__ rows, int H, float eps, int center,
+                                     const float* __restrict__ w2, T2* __restrict__ y2, float eps2, int center2) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const f32x4* xr = (const f32x4*)(x + (size_t)(rows ? rows[r] : r) * H);
+    const f32x4* wr = (const f32x4*)w;
+    T* yr = y + (size_t)r * H;
+    const int nv = H >> 2;
+    f32x4 v[VPT];
+    float sm = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < nv) { v[j] = xr[i]; sm += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]); }
+    }
+    const float mean = center ? block_sum(sm, scratch) / (float)H : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < nv) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[j][e] -= mean; ss += v[j][e] * v[j][e]; }
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)H + eps);
+    float sm2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < nv) {
+            const f32x4 wv = wr[i];
+            if (ADD) {
+                f32x4 acc = ((const f32x4*)yr)[i];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { acc[e] += v[j][e] * inv * wv[e]; v[j][e] = acc[e]; sm2 += acc[e]; }
+                ((f32x4*)yr)[i] = acc;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) yr[4 * i + e] = from_f32<T>(v[j][e] * inv * wv[e]);
+            }
+        }
+    }
+    if (!ADD || !w2) return;
+    // v holds the new residual row: its norm with w2
+    const float mean2 = center2 ? block_sum(sm2, scratch) / (float)H : 0.f;
+    float ss2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < nv) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[j][e] -= mean2; ss2 += v[j][e] * v[j][e]; }
+        }
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum(ss2, scratch) / (float)H + eps2);
+    T2* y2r = y2 + (size_t)r * H;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int i = threadIdx.x + j * blockDim.x;
+        if (i < nv) {
+            const f32x4 wv = ((const f32x4*)w2)[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y2r[4 * i + e] = from_f32<T2>(v[j][e] * inv2 * wv[e]);
+        }
+    }
+}
+
+// `w2`, `y2` (optional, with `add` only): also y2 = norm2(y) of the rows just added to, in `y2`'s dtype.
 extern "C" int br_layernorm(const float* x, const float* w, void* y, int y_is_bf16, const int* rows, int R, int H,
-                            float eps, int center, int add, hipStream_t s) {
+                            float eps, int center, int add, const float* w2, void* y2, int y2_is_bf16, float eps2,
+                            int center2, hipStream_t s) {
     if (R <= 0) return BR_OK;
-    if (H <= 0 || (add && (y_is_bf16 || rows))) return BR_BAD_ARG;
+    if (H <= 0 || (add && (y_is_bf16 || rows)) || (w2 && (!add || !y2))) return BR_BAD_ARG;
     const int threads = H >= 2048 ? 256 : (H >= 512 ? 128 : 64);
+    const bool vec = (H % 4 == 0) && (H / 4 <= 4 * threads) &&
+                     (((uintptr_t)x | (uintptr_t)w | (uintptr_t)y | (uintptr_t)w2 | (uintptr_t)y2) % 16 == 0);
+    if (vec) {
+        if (add) {
+            if (y2_is_bf16) layernorm_vec_kernel<float, bf16, true, 4><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center, w2, (bf16*)y2, eps2, center2);
+            else layernorm_vec_kernel<float, float, true, 4><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center, w2, (float*)y2, eps2, center2);
+        } else if (y_is_bf16) layernorm_vec_kernel<bf16, float, false, 4><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps, center, nullptr, nullptr, 0.f, 0);
+        else layernorm_vec_kernel<float, float, false, 4><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center, nullptr, nullptr, 0.f, 0);
+        return br_check_launch();
+    }
     if (add) layernorm_kernel<float, true><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
     else if (y_is_bf16) layernorm_kernel<bf16, false><<<R, threads, 0, s>>>(x, w, (bf16*)y, rows, H, eps, center);
     else layernorm_kernel<float, false><<<R, threads, 0, s>>>(x, w, (float*)y, rows, H, eps, center);
+    if (w2) {       // widths the one-pass kernel does not take: the second norm as a launch of its own
+        if (y2_is_bf16) layernorm_kernel<bf16, false><<<R, threads, 0, s>>>((const float*)y, w2, (bf16*)y2, nullptr, H, eps2, center2);
+        else layernorm_kernel<float, false><<<R, threads, 0, s>>>((const float*)y, w2, (float*)y2, nullptr, H, eps2, center2);
+    }
     return br_check_launch();
 }
 

@@ -4,112 +4,281 @@
 //     o_t = S_t^T q_t
 // with the forget gate f_t in (lower, 1) per channel deciding what stays and what is written
 // (no key, no further scale).  The columns of S never meet: column c follows
-// S[:, c] <- f * S[:, c] + (1 - f) * v[c], so the work is cut by (sequence, head, 64 columns).
+// S[:, c] <- f * S[:, c] + (1 - f) * v[c], so the work is cut by (sequence, head, 16 columns).
 //
-// Three kernels: `gates` turns the projections' float sums into q = silu(.) and
-// f = lower + (1 - lower) * sigmoid(. + bias) in place (parallel over tokens), `scan` walks a
-// sequence's new tokens in order from the state its slot holds and leaves the state behind,
-// `head_norm` is the RMS norm of every head's output over its e channels.
+// Two kernels: `scan` turns the projections' float sums into q = silu(.) and
+// f = lower + (1 - lower) * sigmoid(. + bias) on their way into LDS and walks a sequence's new
+// tokens in order from the state its slot holds, leaving the state behind; `head_norm` is the RMS
+// norm of every head's output over its e channels.
 #include "common.h"
 
-// ---------------------------------------------------------------------- gates ------
-// rows [T, 2 * hd + he]: q | f | v (hd = heads * d); q and f are rewritten.
-__global__ void glr_gates_kernel(float* __restrict__ rows, const float* __restrict__ f_bias,
-                                 const float* __restrict__ lower, int hd, int width, size_t n) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const size_t t = i / (2 * (size_t)hd);
-    const int c = (int)(i - t * 2 * (size_t)hd);
-    float* r = rows + t * width;
-    const float z = r[c];
-    if (c < hd) r[c] = z / (1.0f + expf(-z));
-    else {
-        const int k = c - hd;
-        const float lo = lower ? lower[k] : 0.f;
-        const float g = 1.0f / (1.0f + expf(-(z + (f_bias ? f_bias[k] : 0.f))));
-        r[c] = lo + (1.0f - lo) * g;
-    }
-}
-
-extern "C" int br_glr_gates(float* rows, const float* f_bias, const float* lower, int T, int hd, int width,
-                            hipStream_t s) {
-    if (T <= 0) return BR_OK;
-    if (hd <= 0 || width < 2 * hd) return BR_BAD_ARG;
-    const size_t n = (size_t)T * 2 * hd;
-    glr_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(rows, f_bias, lower, hd, width, n);
-    return br_check_launch();
-}
-
 // ----------------------------------------------------------------------- scan ------
-// grid (sequences, heads, ceil(e / 64)), 256 threads: thread (c, g) owns column c of the
-// workgroup's 64 and the rows g, g + 4, g + 8, ... of S, RPT of them in registers.  The four
-// row groups' shares of o_t[c] are added in group order through LDS.
-template <int RPT>
+// rows [T, 2 * hd + he] are the projections' float sums q | f | v (hd = heads * d).
+// grid (sequences, heads, ceil(e / 16)), 256 threads.  A workgroup walks its sequence's new tokens for 16
+// columns of one head's state, TC tokens at a time through two LDS stages: while the waves work on one
+// chunk, the next chunk's rows are on their way from memory into registers (coalesced, 16 bytes a thread
+// where rows are aligned so), and go into the other stage with the gates applied (q = silu(.),
+// f = lower + (1 - lower) * sigmoid(. + bias)) behind the chunk's one barrier.  Each wave owns 4 of the 16
+// columns and needs no other barrier: lane (cg, g) holds the rows g RPL .. g RPL + RPL - 1 of column cg in
+// registers; a token costs it RPL / 4 reads of 16 bytes each of gates and queries from LDS (the same for
+// the four columns), one value, 3 RPL multiply-adds and four moves between neighbouring lanes that add the
+// 16 row groups' shares of o_t[c] in a fixed order.  Rows from d to 16 RPL are padding: gate 1, query 0, state 0.
+//
+// A slot's state lies as the lanes hold it: [head][column block of 4][k][lane], S[r][c] at block c / 4,
+// k = r % RPL, lane = 16 (c % 4) + r / RPL, so a wave reads and writes 256 contiguous bytes for each k.
+// The sum of v over each row of 16 lanes, in every lane of the row, by four data-parallel-primitive moves
+// (neighbour, other pair, other quad mirrored, other half mirrored) in a fixed order.
+__device__ __forceinline__ float glr_row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return v;
+}
+
+//
+// LOCAL (the first pass over a long prompt cut into pieces, see `br_glr_scan_pieces`): the state starts at
+// zero, nothing is written to o, and beside the piece's last state the products of its gates go to `decay`
+// ([sequences of the launch][head][16 RPL], in row order).
+template <int RPL, int TC, bool V4, bool LOCAL>
 __global__ __launch_bounds__(256) void glr_scan_kernel(
-    const float* __restrict__ rows, float* __restrict__ o, float* __restrict__ state,
-    const int* __restrict__ cu_seqlens, const int* __restrict__ slots, int H, int d, int e, int width,
-    size_t slot_stride) {
-    __shared__ float part[2][4][64];
-    const int s = blockIdx.x, h = blockIdx.y;
-    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int c = blockIdx.z * 64 + cl;
+    const float* __restrict__ rows, const float* __restrict__ f_bias, const float* __restrict__ lower,
+    float* __restrict__ o, float* __restrict__ state, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, int H, int d, int e, int width, size_t slot_stride, float* __restrict__ decay) {
+    constexpr int DP = RPL * 16;                   // rows of a column with padding
+    constexpr int NL = TC * DP / 1024;             // groups of 4 rows a thread brings per chunk and array
+    extern __shared__ float lds[];
+    float* fL = lds;                               // [2][TC][DP]
+    float* qL = fL + 2 * TC * DP;                  // [2][TC][DP]
+    float* vL = qL + 2 * TC * DP;                  // [2][TC][16]
+    const int s = blockIdx.x, h = blockIdx.y, cb16 = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cg = lane >> 4, g = lane & 15;
+    const int cb4 = cb16 * 4 + wave, c = cb4 * 4 + cg;
     const int slot = slots[s];
     if (slot < 0) return;
     const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
     const bool live = c < e;
-    float* S = state + (size_t)slot * slot_stride + ((size_t)h * d) * e;
-    float st[RPT];
+    const int ncb4 = (e + 3) >> 2;
+    float* S = state + (size_t)slot * slot_stride + (((size_t)h * ncb4 + cb4) * RPL) * 64 + lane;
+    float st[RPL];
 #pragma unroll
-    for (int k = 0; k < RPT; ++k) {
-        const int r = g + 4 * k;
-        st[k] = (live && r < d) ? S[(size_t)r * e + c] : 0.f;
-    }
+    for (int k = 0; k < RPL; ++k) st[k] = (!LOCAL && cb4 < ncb4) ? S[(size_t)k * 64] : 0.f;
+    float dec[LOCAL ? RPL : 1];
+#pragma unroll
+    for (int k = 0; k < (LOCAL ? RPL : 1); ++k) dec[k] = 1.f;
     const int hd = H * d;
-    for (int t = t0; t < t1; ++t) {
-        const float* row = rows + (size_t)t * width;
-        const float* qr = row + h * d;
-        const float* fr = row + hd + h * d;
-        const float vc = live ? row[2 * hd + h * e + c] : 0.f;
-        float sum = 0.f;
+    // what this thread brings per chunk: group i is rows r4 .. r4 + 3 of token tt
+    int l_tt[NL], l_r4[NL];
+    float lo4[NL][4], b4[NL][4];
 #pragma unroll
-        for (int k = 0; k < RPT; ++k) {
-            const int r = g + 4 * k;
-            if (r < d) {
-                const float f = fr[r];
-                st[k] = fmaf(f, st[k], (1.0f - f) * vc);
-                sum = fmaf(st[k], qr[r], sum);
+    for (int i = 0; i < NL; ++i) {
+        const int idx = tid + 256 * i;
+        l_tt[i] = idx / (DP / 4);
+        l_r4[i] = (idx % (DP / 4)) * 4;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int r = l_r4[i] + x;
+            lo4[i][x] = (r < d && lower) ? lower[h * d + r] : 0.f;
+            b4[i][x] = (r < d && f_bias) ? f_bias[h * d + r] : 0.f;
+        }
+    }
+    const int v_tt = tid >> 4, v_c = cb16 * 16 + (tid & 15);
+    float rq[NL][4], rf[NL][4], rv = 0.f;
+
+    auto fetch = [&](int tc0) {                    // rows of the chunk that starts at token tc0, raw, into registers
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int t = tc0 + l_tt[i];
+            const float* qp = rows + (size_t)t * width + h * d + l_r4[i];
+            if (V4) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f}, bq = {0.f, 0.f, 0.f, 0.f};
+                if (t < t1 && l_r4[i] < d) { a = *(const f32x4*)qp; bq = *(const f32x4*)(qp + hd); }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) { rq[i][x] = a[x]; rf[i][x] = bq[x]; }
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const bool ok = t < t1 && l_r4[i] + x < d;
+                    rq[i][x] = ok ? qp[x] : 0.f;
+                    rf[i][x] = ok ? qp[hd + x] : 0.f;
+                }
             }
         }
-        float (*pt)[64] = part[(t - t0) & 1];
-        pt[g][cl] = sum;
-        __syncthreads();
-        if (g == 0 && live)
-            o[(size_t)t * H * e + h * e + c] = ((pt[0][cl] + pt[1][cl]) + pt[2][cl]) + pt[3][cl];
-    }
+        const int t = tc0 + v_tt;
+        rv = (v_tt < TC && t < t1 && v_c < e) ? rows[(size_t)t * width + 2 * hd + h * e + v_c] : 0.f;
+    };
+    auto stage = [&](int buf) {                    // the fetched rows into LDS stage `buf`, gates applied
 #pragma unroll
-    for (int k = 0; k < RPT; ++k) {
-        const int r = g + 4 * k;
-        if (live && r < d) S[(size_t)r * e + c] = st[k];
+        for (int i = 0; i < NL; ++i) {
+            f32x4 qo, fo;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const bool real = l_r4[i] + x < d;
+                // exp and reciprocal by the hardware's own instructions (about an ulp each)
+                const float z = rq[i][x];
+                qo[x] = real ? z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z)) : 0.f;
+                const float gt = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * (rf[i][x] + b4[i][x])));
+                fo[x] = real ? lo4[i][x] + (1.0f - lo4[i][x]) * gt : 1.f;
+            }
+            *(f32x4*)(qL + ((size_t)buf * TC + l_tt[i]) * DP + l_r4[i]) = qo;
+            *(f32x4*)(fL + ((size_t)buf * TC + l_tt[i]) * DP + l_r4[i]) = fo;
+        }
+        if (v_tt < TC) vL[(buf * TC + v_tt) * 16 + (tid & 15)] = rv;
+    };
+
+    fetch(t0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    float* orow = o + (size_t)t0 * H * e + h * e + c;
+    for (int tc0 = t0; tc0 < t1; tc0 += TC) {
+        const bool more = tc0 + TC < t1;
+        if (more) fetch(tc0 + TC);
+        const int nt = t1 - tc0 < TC ? t1 - tc0 : TC;
+        // the next token's gates, queries and value are asked from LDS before this token's are used
+        const float* fp = fL + (size_t)buf * TC * DP + g * RPL;
+        const float* qp = qL + (size_t)buf * TC * DP + g * RPL;
+        const float* vp = vL + buf * TC * 16 + wave * 4 + cg;
+        f32x4 fc[RPL / 4], qc[RPL / 4];
+        float vc = vp[0];
+#pragma unroll
+        for (int k4 = 0; k4 < RPL / 4; ++k4) { fc[k4] = *(const f32x4*)(fp + 4 * k4); qc[k4] = *(const f32x4*)(qp + 4 * k4); }
+        for (int tt = 0; tt < nt; ++tt) {
+            const int nx = tt + 1 < TC ? tt + 1 : tt;
+            f32x4 fn[RPL / 4], qn[RPL / 4];
+            const float vn = vp[nx * 16];
+#pragma unroll
+            for (int k4 = 0; k4 < RPL / 4; ++k4) {
+                fn[k4] = *(const f32x4*)(fp + (size_t)nx * DP + 4 * k4);
+                qn[k4] = *(const f32x4*)(qp + (size_t)nx * DP + 4 * k4);
+            }
+            float sum = 0.f;
+#pragma unroll
+            for (int k4 = 0; k4 < RPL / 4; ++k4) {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    // f s + (1 - f) v as v + f (s - v): a subtraction and a multiply-add a row
+                    st[4 * k4 + x] = fmaf(fc[k4][x], st[4 * k4 + x] - vc, vc);
+                    if (LOCAL) dec[LOCAL ? 4 * k4 + x : 0] *= fc[k4][x];
+                    else sum = fmaf(st[4 * k4 + x], qc[k4][x], sum);
+                }
+            }
+            if (!LOCAL) {
+                sum = glr_row16_sum(sum);
+                if (g == 0 && live) orow[0] = sum;
+                orow += (size_t)H * e;
+            }
+            vc = vn;
+#pragma unroll
+            for (int k4 = 0; k4 < RPL / 4; ++k4) { fc[k4] = fn[k4]; qc[k4] = qn[k4]; }
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    if (cb4 < ncb4) {
+#pragma unroll
+        for (int k = 0; k < RPL; ++k) S[(size_t)k * 64] = st[k];
+    }
+    if (LOCAL && cb16 == 0 && wave == 0 && cg == 0) {
+        float* dr = decay + ((size_t)s * H + h) * DP + g * RPL;
+#pragma unroll
+        for (int k = 0; k < (LOCAL ? RPL : 1); ++k) dr[k] = dec[k];
     }
 }
 
-// `slot_stride`: floats from one slot's state to the next (at least H * d * e).
-extern "C" int br_glr_scan(const float* rows, float* o, float* state, const int* cu_seqlens, const int* slots,
-                           int B, int H, int d, int e, int width, size_t slot_stride, hipStream_t s) {
-    if (B <= 0) return BR_OK;
-    if (H <= 0 || H > 65535 || d <= 0 || e <= 0 || d > 512 || width < 2 * H * d + H * e ||
-        slot_stride < (size_t)H * d * e)
+// Between the two passes over a prompt cut into `pieces` pieces per sequence: from the sequence's own state
+// s_0 and every piece's local last state L_c and gate products D_c, the state each piece starts from,
+// s_(c+1) = D_c s_c + L_c, written over L_c; the last one becomes the sequence's state.
+// grid (sequences, heads * column blocks of 4), block 64.
+__global__ __launch_bounds__(64) void glr_carry_kernel(float* __restrict__ state, size_t slot_stride,
+                                                       const int* __restrict__ slots, float* __restrict__ piece_state,
+                                                       size_t piece_stride, const float* __restrict__ decay, int pieces,
+                                                       int H, int ncb4, int rpl) {
+    const int b = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x;
+    const int slot = slots[b];
+    if (slot < 0) return;
+    const int h = hc / ncb4, dp = rpl * 16;
+    for (int k = 0; k < rpl; ++k) {
+        const size_t idx = ((size_t)hc * rpl + k) * 64 + lane;
+        const int r = (lane & 15) * rpl + k;
+        float sv = state[(size_t)slot * slot_stride + idx];
+        for (int c = 0; c < pieces; ++c) {
+            const size_t v = (size_t)b * pieces + c;
+            const float local = piece_state[v * piece_stride + idx];
+            piece_state[v * piece_stride + idx] = sv;
+            sv = fmaf(decay[(v * H + h) * dp + r], sv, local);
+        }
+        state[(size_t)slot * slot_stride + idx] = sv;
+    }
+}
+
+// Rows a lane holds for a head of d query channels: ceil(d / 16) rounded up to 4, 8, 16 or 32.
+static inline int glr_rpl(int d) {
+    const int r = (d + 15) / 16;
+    return r <= 4 ? 4 : (r <= 8 ? 8 : (r <= 16 ? 16 : 32));
+}
+extern "C" int br_glr_rows_per_lane(int d) { return glr_rpl(d); }
+
+template <bool LOCAL>
+static int glr_scan_launch(const float* rows, const float* f_bias, const float* lower, float* o, float* state,
+                           const int* cu_seqlens, const int* slots, int B, int H, int d, int e, int width,
+                           size_t slot_stride, float* decay, hipStream_t s) {
+    const int ncb4 = (e + 3) / 4, rpl = glr_rpl(d);
+    if (H <= 0 || H > 65535 || d <= 0 || e <= 0 || d > 512 || (e + 15) / 16 > 65535 || width < 2 * H * d + H * e ||
+        slot_stride < (size_t)H * ncb4 * rpl * 64 || (LOCAL && !decay))
         return BR_BAD_ARG;
-    dim3 grid(B, H, (e + 63) / 64);
-    const int rpt = (d + 3) / 4;
-#define GLR_SCAN(R) glr_scan_kernel<R><<<grid, 256, 0, s>>>(rows, o, state, cu_seqlens, slots, H, d, e, width, slot_stride)
-    if (rpt <= 8) GLR_SCAN(8);
-    else if (rpt <= 16) GLR_SCAN(16);
-    else if (rpt <= 32) GLR_SCAN(32);
-    else if (rpt <= 64) GLR_SCAN(64);
-    else GLR_SCAN(128);
+    dim3 grid(B, H, (e + 15) / 16);
+    // 16-byte loads where every row piece starts at a multiple of 16 bytes
+    const bool v4 = d % 4 == 0 && width % 4 == 0 && ((uintptr_t)rows % 16) == 0;
+#define GLR_SCAN(R, TC) do { \
+        const size_t lds = (size_t)(4 * TC * R * 16 + 2 * TC * 16) * sizeof(float); \
+        if (v4) glr_scan_kernel<R, TC, true, LOCAL><<<grid, 256, lds, s>>>(rows, f_bias, lower, o, state, cu_seqlens, slots, H, d, e, width, slot_stride, decay); \
+        else glr_scan_kernel<R, TC, false, LOCAL><<<grid, 256, lds, s>>>(rows, f_bias, lower, o, state, cu_seqlens, slots, H, d, e, width, slot_stride, decay); \
+    } while (0)
+    if (rpl == 4) GLR_SCAN(4, 16);
+    else if (rpl == 8) GLR_SCAN(8, 16);
+    else if (rpl == 16) GLR_SCAN(16, 16);
+    else GLR_SCAN(32, 8);
 #undef GLR_SCAN
     return br_check_launch();
+}
+
+// `slot_stride`: floats from one slot's state to the next (at least H * ceil(e / 4) * rows per lane * 64).
+extern "C" int br_glr_scan(const float* rows, const float* f_bias, const float* lower, float* o, float* state,
+                           const int* cu_seqlens, const int* slots, int B, int H, int d, int e, int width,
+                           size_t slot_stride, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    return glr_scan_launch<false>(rows, f_bias, lower, o, state, cu_seqlens, slots, B, H, d, e, width, slot_stride, nullptr, s);
+}
+
+// A step of long prompts with every sequence cut into `pieces` pieces that run side by side: the recurrence is
+// linear in the state, so a piece can be walked from a zero state first (its last state L and the products D of
+// its gates), the pieces' true first states follow from s_(c+1) = D_c s_c + L_c, and a second walk from those
+// writes o.  Twice the arithmetic for `pieces` times the workgroups; results differ from the plain walk by the
+// rounding of that one combination per piece.  `piece_cu` [B * pieces + 1] cuts the packed tokens (pieces of a
+// sequence in order, empty ones allowed), `piece_slots` [B * pieces] is the piece's own number (or -1 for a
+// padding sequence's), `piece_state` [B * pieces][state of a slot] and `decay` [B * pieces][H][16 * rows per lane]
+// are scratch.
+extern "C" int br_glr_scan_pieces(const float* rows, const float* f_bias, const float* lower, float* o, float* state,
+                                  const int* slots, const int* piece_cu, const int* piece_slots, float* piece_state,
+                                  float* decay, int B, int pieces, int H, int d, int e, int width, size_t slot_stride,
+                                  hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (pieces <= 0 || (long long)B * pieces > 65535) return BR_BAD_ARG;
+    const int ncb4 = (e + 3) / 4, rpl = glr_rpl(d);
+    const size_t piece_stride = (size_t)H * ncb4 * rpl * 64;
+    int rc = glr_scan_launch<true>(rows, f_bias, lower, o, piece_state, piece_cu, piece_slots, B * pieces, H, d, e, width,
+                                   piece_stride, decay, s);
+    if (rc != BR_OK) return rc;
+    if ((long long)H * ncb4 > 65535) return BR_BAD_ARG;
+    glr_carry_kernel<<<dim3(B, H * ncb4), 64, 0, s>>>(state, slot_stride, slots, piece_state, piece_stride, decay, pieces, H,
+                                                      ncb4, rpl);
+    rc = br_check_launch();
+    if (rc != BR_OK) return rc;
+    return glr_scan_launch<false>(rows, f_bias, lower, o, piece_state, piece_cu, piece_slots, B * pieces, H, d, e, width,
+                                  piece_stride, nullptr, s);
 }
 
 // ------------------------------------------------------------------ head norm ------

@@ -11,12 +11,13 @@
 // Three kernels: `prepare` (bias, per-head RMS norm of queries and keys, rotation of the
 // first `rd` elements in (i, i + rd/2) pairs, value mixing with another layer's values,
 // cache write), `pool` (the means of the blocks that the step completed) and `attend`.
-// Keys and values of a page: [kv_head][token][dk] and, behind the keys of all heads,
-// [kv_head][token][dv].
+// Keys and values of a page: keys [kv_head][token][dk] and, behind the keys of all heads, values
+// transposed, [kv_head][dv][token]: the operand layout of the matrix-core kernel below (a lane reads
+// 8 consecutive tokens of one value channel).
 //
-// The sums of `attend` run over the seen blocks in ascending order and then over the window's
-// tokens in ascending position, 64 at a time, so the chunking depends on (p, size, pool) only:
-// whole prompts, portions and single tokens give the same bits.
+// The sums of `attend` run over the pages of the seen blocks and then over the pages of the window's
+// tokens, so the order depends on (p, size, pool) only: whole prompts, portions and single tokens give
+// the same bits.
 #include "common.h"
 
 #define MAX_EPL 8   // head widths up to 64 * MAX_EPL
@@ -51,8 +52,9 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
         const int pg = block_table[(size_t)slot * table_stride + p / page];
         T* pb = storage + (size_t)pg * page_elems;
         dst = is_k ? pb + ((size_t)kvh * page + (p % page)) * dk
-                   : pb + (size_t)nkv * page * dk + ((size_t)kvh * page + (p % page)) * dv;
+                   : pb + (size_t)nkv * page * dk + (size_t)kvh * dv * page + (p % page);
     }
+    const int dst_step = (is_q || is_k) ? 1 : page;      // values lie transposed: channel i of a token at i * page
     float v[MAX_EPL];
     float ss = 0.f;
 #pragma unroll
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
 #pragma unroll
         for (int j = 0; j < MAX_EPL; ++j) {
             const int i = lane + 64 * j;
-            if (i < n) dst[i] = from_f32<T>(v[j]);
+            if (i < n) dst[(size_t)i * dst_step] = from_f32<T>(v[j]);
         }
     }
 }
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(
     const int* bt = block_table + (size_t)slot * table_stride;
     const int ppg = pooled_table[(size_t)slot * pooled_stride + b / page];
     T* pk = pooled + (size_t)ppg * page_elems + ((size_t)kvh * page + (b % page)) * dk;
-    T* pv = pooled + (size_t)ppg * page_elems + (size_t)nkv * page * dk + ((size_t)kvh * page + (b % page)) * dv;
+    T* pv = pooled + (size_t)ppg * page_elems + (size_t)nkv * page * dk + (size_t)kvh * dv * page + (b % page);
     const float inv = 1.0f / (float)pool;
     for (int i = lane; i < dk + dv; i += 64) {
         const bool key = i < dk;
@@ -167,10 +169,10 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(
             const int j = b * pool + r;
             const T* pb = storage + (size_t)bt[j / page] * page_elems;
             acc += key ? to_f32<T>(pb[((size_t)kvh * page + (j % page)) * dk + i])
-                       : to_f32<T>(pb[(size_t)nkv * page * dk + ((size_t)kvh * page + (j % page)) * dv + (i - dk)]);
+                       : to_f32<T>(pb[(size_t)nkv * page * dk + ((size_t)kvh * dv + (i - dk)) * page + (j % page)]);
         }
         if (key) pk[i] = from_f32<T>(acc * inv);
-        else pv[i - dk] = from_f32<T>(acc * inv);
+        else pv[(size_t)(i - dk) * page] = from_f32<T>(acc * inv);
     }
 }
 
@@ -194,86 +196,135 @@ extern "C" int br_pwa_pool(const void* storage, const int* block_table, int tabl
 }
 
 // -------------------------------------------------------------------- attend -------
-// One wave per (query token, query head).  Key c of a query: pooled row c for c < nb, the token
-// lo + c - nb after that.  Online softmax (m' = max(m, s), corr = exp(m - m'), l = l corr + sum w,
-// acc = acc corr + w v); a sink starts it at m = 0, l = 1 instead of m = -inf, l = 0.
-template <typename T>
-__global__ __launch_bounds__(64) void pwa_attend_kernel(
+// One workgroup of four waves per (query token, query head), float arithmetic.  The query's keys come a
+// page at a time: first the pages of the pooled unit that hold rows 0 .. seen - 1, then the token pages
+// from the one that holds lo to the one that holds p; rows outside what the query sees are masked.  Page
+// number n of that list is wave n % 4's.  A lane scores one row of the page (16 bytes a load where the
+// width allows it), the wave takes an online-softmax step (m' = max(m, s), corr = exp(m - m'),
+// l = l corr + sum w, acc = acc corr + w v), and in the second product a lane owns value channels and
+// reads 8 neighbouring rows of a channel at a time from the transposed values.  The four waves' (m, l, acc)
+// are merged in wave order at the end.  A sink starts wave 0 at m = 0, l = 1 instead of m = -inf, l = 0.
+// Which page goes to which wave depends on (p, size, pool) only: whole prompts, portions and single
+// tokens give the same bits.
+template <typename T> struct pwa_vec;
+template <> struct pwa_vec<float> { static constexpr int N = 4; typedef f32x4 type; };
+template <> struct pwa_vec<bf16> { static constexpr int N = 8; typedef bf16x8 type; };
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void pwa_attend_kernel(
     const T* __restrict__ q, T* __restrict__ out, const int* __restrict__ pos,
     const int* __restrict__ seq_of_token, const int* __restrict__ slots,
     const int* __restrict__ block_table, int table_stride, const T* __restrict__ storage,
     const int* __restrict__ pooled_table, int pooled_stride, const T* __restrict__ pooled,
     int nq, int nkv, int dk, int dv, int page, int size, int pool, float scale, int sink) {
     extern __shared__ float lds[];
-    float* qs = lds;            // [dk]
-    float* ps = lds + dk;       // [64]
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float* qs = lds;                         // [dk]
+    float* ps = qs + dk;                     // [4][64]
+    float* ml = ps + 256;                    // [4][2]
+    float* accs = ml + 8;                    // [4][dv]
+    constexpr int VN = pwa_vec<T>::N;
+    typedef typename pwa_vec<T>::type vec_t;
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int kvh = h / (nq / nkv);
     T* o = out + ((size_t)t * nq + h) * dv;
     const int slot = slots[seq_of_token[t]];
     if (slot < 0) {
-        for (int d = lane; d < dv; d += 64) o[d] = from_f32<T>(0.f);
+        for (int d = threadIdx.x; d < dv; d += 256) o[d] = from_f32<T>(0.f);
         return;
     }
     const T* qr = q + ((size_t)t * nq + h) * dk;
-    for (int d = lane; d < dk; d += 64) qs[d] = to_f32<T>(qr[d]);
+    for (int d = threadIdx.x; d < dk; d += 256) qs[d] = to_f32<T>(qr[d]);
     __syncthreads();
     const int p = pos[t];
-    const int lo = (size > 0 && p - size + 1 > 0) ? p - size + 1 : 0;
-    int nb = 0;
-    if (pool > 0 && size > 0 && p - size - pool + 1 >= 0) nb = (p - size - pool + 1) / pool + 1;
-    const int total = nb + (p - lo + 1);
+    const int lo = (p - size + 1 > 0) ? p - size + 1 : 0;
+    int seen = 0;
+    if (pool > 0 && p - size - pool + 1 >= 0) seen = (p - size - pool + 1) / pool + 1;
+    const int far_pages = (seen + page - 1) / page;
+    const int first_page = lo / page, n_pages = far_pages + p / page - first_page + 1;
     const int* bt = block_table + (size_t)slot * table_stride;
     const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
     const size_t page_elems = (size_t)nkv * page * (dk + dv);
-    const size_t k_off = (size_t)kvh * page * dk, v_off = (size_t)nkv * page * dk + (size_t)kvh * page * dv;
+    const size_t k_off = (size_t)kvh * page * dk, v_off = (size_t)nkv * page * dk + (size_t)kvh * dv * page;
+    float* pw = ps + wave * 64;
 
-    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+    float m = (sink && wave == 0) ? 0.f : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
     float acc[MAX_EPL];
 #pragma unroll
     for (int i = 0; i < MAX_EPL; ++i) acc[i] = 0.f;
 
-    for (int c0 = 0; c0 < total; c0 += 64) {
-        const int c = c0 + lane;
+    for (int n = wave; n < n_pages; n += 4) {
+        const bool far = n < far_pages;
+        const int pi = far ? n : first_page + (n - far_pages);         // page index within its unit
+        const T* base = far ? pooled + (size_t)pt[pi] * page_elems : storage + (size_t)bt[pi] * page_elems;
+        const int row0 = pi * page;                                    // first row of the page
+        const int first_ok = far ? 0 : lo, last_ok = far ? seen - 1 : p;
         float s = -INFINITY;
-        if (c < total) {
-            const bool pl = c < nb;
-            const int j = pl ? c : lo + (c - nb);
-            const T* base = pl ? pooled + (size_t)pt[j / page] * page_elems : storage + (size_t)bt[j / page] * page_elems;
-            const T* kr = base + k_off + (size_t)(j % page) * dk;
-            float dot = 0.f;
-            for (int d = 0; d < dk; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
-            s = dot * scale;
-        }
-        const float m_new = fmaxf(m, wave_max(s));
-        const float corr = expf(m - m_new);          // exp(-inf) = 0 on the first chunk without a sink
-        const float w = (c < total) ? expf(s - m_new) : 0.f;
-        l = l * corr + wave_sum(w);
-        __syncthreads();
-        ps[lane] = w;
-        __syncthreads();
-        const int nk = (total - c0) < 64 ? (total - c0) : 64;
+        for (int j = lane; j < page; j += 64) {                       // pages of 64 rows: one row a lane
+            const int key = row0 + j;
+            if (key >= first_ok && key <= last_ok) {
+                const T* kr = base + k_off + (size_t)j * dk;
+                float dot = 0.f;
+                if (VEC) {
+                    for (int d = 0; d < dk; d += VN) {
+                        const vec_t kv = *(const vec_t*)(kr + d);
 #pragma unroll
-        for (int i = 0; i < MAX_EPL; ++i) acc[i] *= corr;
-        for (int jj = 0; jj < nk; ++jj) {
-            const int cc = c0 + jj;
-            const bool pl = cc < nb;
-            const int j = pl ? cc : lo + (cc - nb);
-            const T* base = pl ? pooled + (size_t)pt[j / page] * page_elems : storage + (size_t)bt[j / page] * page_elems;
-            const T* vr = base + v_off + (size_t)(j % page) * dv;
-            const float pw = ps[jj];
-#pragma unroll
-            for (int i = 0; i < MAX_EPL; ++i) {
-                const int d = lane + 64 * i;
-                if (d < dv) acc[i] = fmaf(pw, to_f32<T>(vr[d]), acc[i]);
+                        for (int i = 0; i < VN; ++i) dot = fmaf(qs[d + i], to_f32<T>(kv[i]), dot);
+                    }
+                } else {
+                    for (int d = 0; d < dk; ++d) dot = fmaf(qs[d], to_f32<T>(kr[d]), dot);
+                }
+                s = dot * scale;
             }
         }
+        const float m_new = fmaxf(m, wave_max(s));
+        if (m_new == -INFINITY) continue;                              // no row of this page is seen (wave-uniform)
+        const float corr = expf(m - m_new);                            // exp(-inf) = 0 on a wave's first page
+        const float w = expf(s - m_new);                               // 0 for masked rows
+        l = l * corr + wave_sum(w);
+        pw[lane] = w;
         m = m_new;
+        // rows of this page that take part: [j_lo, j_hi)
+        const int j_lo = first_ok > row0 ? first_ok - row0 : 0;
+        const int j_hi = last_ok - row0 + 1 < page ? last_ok - row0 + 1 : page;
+#pragma unroll
+        for (int i = 0; i < MAX_EPL; ++i) {
+            const int d = lane + 64 * i;
+            if (d < dv) {
+                const T* vr = base + v_off + (size_t)d * page;
+                float a = acc[i] * corr;
+                if (VEC) {
+                    for (int j = (j_lo / VN) * VN; j < j_hi; j += VN) {
+                        const vec_t vv = *(const vec_t*)(vr + j);
+#pragma unroll
+                        for (int e = 0; e < VN; ++e)
+                            if (j + e >= j_lo && j + e < j_hi) a = fmaf(pw[j + e], to_f32<T>(vv[e]), a);
+                    }
+                } else {
+                    for (int j = j_lo; j < j_hi; ++j) a = fmaf(pw[j], to_f32<T>(vr[j]), a);
+                }
+                acc[i] = a;
+            }
+        }
     }
+    if (lane == 0) { ml[2 * wave] = m; ml[2 * wave + 1] = l; }
 #pragma unroll
     for (int i = 0; i < MAX_EPL; ++i) {
         const int d = lane + 64 * i;
-        if (d < dv) o[d] = from_f32<T>(acc[i] / l);
+        if (d < dv) accs[wave * dv + d] = acc[i];
+    }
+    __syncthreads();
+    float M = fmaxf(fmaxf(ml[0], ml[2]), fmaxf(ml[4], ml[6]));
+    float L = 0.f, c4[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        c4[w] = ml[2 * w] == -INFINITY ? 0.f : expf(ml[2 * w] - M);
+        L += ml[2 * w + 1] * c4[w];
+    }
+    for (int d = threadIdx.x; d < dv; d += 256) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) a += accs[w * dv + d] * c4[w];
+        o[d] = from_f32<T>(a / L);
     }
 }
 
@@ -282,18 +333,226 @@ extern "C" int br_pwa_attend(const void* q, void* out, int is_bf16, const int* p
                              const int* pooled_table, int pooled_stride, const void* pooled, int T, int nq, int nkv,
                              int dk, int dv, int page, int size, int pool, float scale, int sink, hipStream_t s) {
     if (T <= 0) return BR_OK;
-    if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL || page <= 0 ||
-        size < 0 || pool < 0 || nq > 65535 || (pool > 0 && size > 0 && (!pooled_table || !pooled)))
+    if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL || page != 64 ||
+        size <= 0 || pool < 0 || nq > 65535 || (pool > 0 && (!pooled_table || !pooled)))
         return BR_BAD_ARG;
     dim3 grid(T, nq);
-    const size_t lds = (size_t)(dk + 64) * sizeof(float);
-    if (is_bf16)
-        pwa_attend_kernel<bf16><<<grid, 64, lds, s>>>((const bf16*)q, (bf16*)out, pos, seq_of_token, slots, block_table,
-                                                      table_stride, (const bf16*)storage, pooled_table, pooled_stride,
-                                                      (const bf16*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink);
-    else
-        pwa_attend_kernel<float><<<grid, 64, lds, s>>>((const float*)q, (float*)out, pos, seq_of_token, slots, block_table,
-                                                       table_stride, (const float*)storage, pooled_table, pooled_stride,
-                                                       (const float*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink);
+    const size_t lds = (size_t)(dk + 256 + 8 + 4 * dv) * sizeof(float);
+    // 16-byte loads where every row starts at a multiple of 16 bytes
+    const bool vec = is_bf16 ? dk % 8 == 0 : dk % 4 == 0;
+#define PWA_ATT(TT, V) pwa_attend_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)q, (TT*)out, pos, seq_of_token, slots, block_table, \
+        table_stride, (const TT*)storage, pooled_table, pooled_stride, (const TT*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink)
+    if (is_bf16) { if (vec) PWA_ATT(bf16, true); else PWA_ATT(bf16, false); }
+    else { if (vec) PWA_ATT(float, true); else PWA_ATT(float, false); }
+#undef PWA_ATT
     return br_check_launch();
+}
+
+// ------------------------------------------------- prompts on the matrix cores -----
+// bfloat16, pages of 64 rows, steps of several tokens per sequence.  grid = (row tiles of 128, nkv,
+// sequences), block = 256.  A row is a (token, query head of the kv head's group) pair, row = token * G
+// + head; each wave owns 32 rows and walks first the pooled rows, then the token rows its queries can
+// see, 32 keys at a time.  Scores are computed transposed, S^T = K Q^T (v_mfma_f32_32x32x16_bf16, float
+// sums), with the block's keys as the product's rows in a fixed permutation such that a lane's 16
+// accumulators are 2 x 8 consecutive keys of its one query column: after the softmax step (float, base
+// 2, the scale folded into the exponent) and rounding they are the B operand of O^T = V^T P^T as they
+// stand, and V^T is read 16 contiguous bytes a lane from the transposed values.  NBK = ceil(dk / 32),
+// NBV = ceil(dv / 32) (rounded up to a size that is compiled; surplus fragments are zero).
+#define PWA_PAGE 64
+#define PWA_LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ bf16x8 pwa_zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+    return z;
+}
+// 8 values V^T[channel][k .. k+7] of a page; rows at or beyond `limit` (not written yet) read as zero
+__device__ __forceinline__ bf16x8 pwa_load_vt8(const bf16* __restrict__ vrow, int k, int limit) {
+    bf16x8 v = *(const bf16x8*)(vrow + k);
+    if (k + 8 > limit) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) if (k + i >= limit) v[i] = (bf16)0.f;
+    }
+    return v;
+}
+// Row c (0..31) of a score block stands for this key of the block; lane (column, g) then holds in
+// acc[r] the key 16 (r / 8) + 8 g + r % 8.
+__device__ __forceinline__ int pwa_key_of_row(int c) { return 16 * (c >> 4) + 8 * ((c >> 2) & 1) + 4 * ((c >> 3) & 1) + (c & 3); }
+
+// One block of 32 keys (rows kb .. kb + 31 of a unit, kl = kb % 64 within the page `pg`): a key is
+// seen by this lane's query if first_ok <= key <= last_ok.
+template <int NBK, int NBV>
+__device__ __forceinline__ void pwa_block(const bf16* __restrict__ pg, size_t k_off, size_t v_off, int kb, int kl,
+                                          int limit, int first_ok, int last_ok, int dk, int dv, int c, int g,
+                                          const bf16x8* qf, f32x16* acc_o, float& m, float& lsum, float scale2) {
+    const bf16* krow = pg + k_off + (size_t)(kl + pwa_key_of_row(c)) * dk;
+    f32x16 s_acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 2 * NBK; ++s) {
+        const int d = s * 16 + 8 * g;
+        const bf16x8 kf = (d < dk) ? *(const bf16x8*)(krow + d) : pwa_zero8();
+        s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], s_acc, 0, 0, 0);
+    }
+    float sv[16];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+        sv[r] = (key >= first_ok && key <= last_ok) ? s_acc[r] * scale2 : -INFINITY;
+        mx = fmaxf(mx, sv[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m - m_use);
+    float psum = 0.f;
+    bf16x8 p1, p2;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(sv[r] - m_use);
+        psum += p;
+        if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
+    }
+    lsum = lsum * corr + psum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+        const int ch = i * 32 + c;
+        bf16x8 v1 = pwa_zero8(), v2 = pwa_zero8();
+        if (ch < dv) {
+            const bf16* vrow = pg + v_off + (size_t)ch * PWA_PAGE;
+            v1 = pwa_load_vt8(vrow, kl + 8 * g, limit);
+            v2 = pwa_load_vt8(vrow, kl + 16 + 8 * g, limit);
+        }
+        acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
+        acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
+    }
+}
+
+template <int NBK, int NBV>
+__global__ __launch_bounds__(256) void pwa_prefill_kernel(
+    const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
+    int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
+    const int G = nq / nkv;
+    const int rows_total = n_new * G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row0 = blockIdx.x * 128 + wave * 32;
+    if (row0 >= rows_total) return;
+    const int c = lane & 31, g = lane >> 5;
+    const int row = row0 + c;
+    const bool row_ok = row < rows_total;
+    const int rr = row_ok ? row : rows_total - 1;
+    const int tok = rr / G, head = kvh * G + rr % G;
+    bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * dv;
+    if (slot < 0) {       // padding: no cache behind it
+        if (row_ok && g == 0) for (int d = 0; d < dv; ++d) orow[d] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], start = ctx - n_new;
+    const int pq = start + tok;
+    const int pq_min = start + row0 / G;
+    const int last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
+    const int pq_max = start + last_row / G;
+
+    const bf16* qrow = q + ((size_t)(t0 + tok) * nq + head) * dk;
+    bf16x8 qf[2 * NBK];
+#pragma unroll
+    for (int s = 0; s < 2 * NBK; ++s) {
+        const int d = s * 16 + 8 * g;
+        qf[s] = (d < dk) ? *(const bf16x8*)(qrow + d) : pwa_zero8();
+    }
+    f32x16 acc_o[NBV];
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    // the two lane halves of a query add their sums at the end: the sink's one goes to the first
+    float m = sink ? 0.f : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
+    const float scale2 = scale * PWA_LOG2E;
+    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
+    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+
+    if (pool > 0) {
+        // blocks wholly before the window: query p sees the pooled rows 0 .. seen(p) - 1
+        const int far_max = pq_max - size - pool + 1, far = pq - size - pool + 1;
+        const int seen_max = far_max >= 0 ? far_max / pool + 1 : 0;
+        const int seen = (row_ok && far >= 0) ? far / pool + 1 : 0;
+        const int written = ctx / pool;
+        const int* pt = pooled_table + (size_t)slot * pooled_stride;
+        for (int kb = 0; kb < seen_max; kb += 32) {
+            const int kl = kb % PWA_PAGE;
+            const bf16* pg = pooled + (size_t)pt[kb / PWA_PAGE] * page_elems;
+            pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, written - (kb - kl), 0, seen - 1, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+        }
+    }
+    const int* bt = block_table + (size_t)slot * table_stride;
+    int lo = pq_min - size + 1;
+    if (lo < 0) lo = 0;
+    const int first_ok = row_ok ? pq - size + 1 : 1, last_ok = row_ok ? pq : 0;
+    for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
+        const int kl = kb % PWA_PAGE;
+        const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
+        pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, ctx - (kb - kl), first_ok, last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!row_ok) return;
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;      // acc_o[i][4 r4 + e]: channel d + e
+            if (d < dv) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc_o[i][4 * r4 + e] * inv);
+                *(bf16x4*)(orow + d) = o;
+            }
+        }
+}
+
+template <int NBK>
+static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
+                                const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
+                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+#define PWA_GO(V) pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink)
+    if (nbv <= 1) PWA_GO(1);
+    else if (nbv <= 2) PWA_GO(2);
+    else if (nbv <= 3) PWA_GO(3);
+    else if (nbv <= 4) PWA_GO(4);
+    else PWA_GO(8);
+#undef PWA_GO
+    return br_check_launch();
+}
+
+// Takes bfloat16, widths of keys in steps of 8 and of values in steps of 4, each up to 256.
+extern "C" int br_pwa_prefill_bf16(const void* q, void* out, const int* cu_seqlens, const int* slots, const int* ctx_lens,
+                                   const int* block_table, int table_stride, const void* storage, const int* pooled_table,
+                                   int pooled_stride, const void* pooled, int B, int max_new, int nq, int nkv, int dk, int dv,
+                                   int size, int pool, float scale, int sink, hipStream_t s) {
+    if (B <= 0 || max_new <= 0) return BR_OK;
+    if (nq <= 0 || nkv <= 0 || nq % nkv || nkv > 65535 || B > 65535 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 ||
+        dv % 4 || size <= 0 || pool < 0 || (pool > 0 && (!pooled_table || !pooled)))
+        return BR_BAD_ARG;
+    const int G = nq / nkv;
+    dim3 grid((unsigned)(((size_t)max_new * G + 127) / 128), nkv, B);
+    const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
+#define PWA_K(KK) pwa_prefill_launch_v<KK>(nbv, grid, s, (const bf16*)q, (bf16*)out, cu_seqlens, slots, ctx_lens, block_table, table_stride, \
+                                           (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink)
+    if (nbk <= 1) return PWA_K(1);
+    if (nbk <= 2) return PWA_K(2);
+    if (nbk <= 3) return PWA_K(3);
+    if (nbk <= 4) return PWA_K(4);
+    return PWA_K(8);
+#undef PWA_K
 }

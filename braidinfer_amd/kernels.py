@@ -110,8 +110,10 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float,
 
 
 def layernorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None,
-              center: bool = True, add: bool = False) -> None:
-    """out = norm(x) * w, or out += norm(x) * w with `add` (float `out`); `center` False: the RMS norm."""
+              center: bool = True, add: bool = False, then=None) -> None:
+    """out = norm(x) * w, or out += norm(x) * w with `add` (float `out`); `center` False: the RMS norm.
+    `then` = (w2, out2, eps2, center2), with `add` only: the rows just added to are normed once more,
+    out2 = norm2(out) * w2, in the same kernel."""
     _dev("layernorm", x, w, out, rows)
     H = x.shape[-1]
     R = out.shape[0]
@@ -123,9 +125,19 @@ def layernorm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, eps: float, r
         _req(rows.dtype == torch.int32 and rows.numel() == R, "layernorm: rows must be int32 [R]")
     _req(not add or (out.dtype == torch.float32 and rows is None and out.data_ptr() != x.data_ptr()),
          "layernorm: adding needs float rows of their own, without a gather")
-    f = _fn("elementwise", "br_layernorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, c_int, c_int, _P])
+    w2 = out2 = None
+    eps2, center2 = 0.0, False
+    if then is not None:
+        w2, out2, eps2, center2 = then
+        _dev("layernorm", w2, out2)
+        _req(add and w2.dtype == torch.float32 and w2.numel() == H and out2.shape == (R, H)
+             and out2.data_ptr() not in (x.data_ptr(), out.data_ptr()), "layernorm: the second norm takes float weights [H] "
+             "and rows [R, H] of their own, behind an add")
+    f = _fn("elementwise", "br_layernorm", [_P, _P, _P, c_int, _P, c_int, c_int, c_float, c_int, c_int, _P, _P, c_int,
+                                            c_float, c_int, _P])
     _check(f(_ptr(x), _ptr(w), _ptr(out), _is_bf16(out, "layernorm"), _ptr(rows), R, H, float(eps), int(center),
-             int(add), _stream()), "layernorm")
+             int(add), _ptr(w2), _ptr(out2), _is_bf16(out2, "layernorm") if out2 is not None else 0, float(eps2),
+             int(center2), _stream()), "layernorm")
 
 
 def scale_(x: torch.Tensor, scale: float) -> None:
@@ -586,34 +598,99 @@ def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_
              int(pool), float(scale), int(sink), _stream()), "pwa_attend")
 
 
+def pwa_prefill_takes(dtype: torch.dtype, dk: int, dv: int, page: int) -> bool:
+    """Whether the matrix-core kernel takes these sizes (else `pwa_attend` does the step)."""
+    return dtype == torch.bfloat16 and page == 64 and dk % 8 == 0 and dv % 4 == 0 and 0 < dk <= 256 and 0 < dv <= 256
+
+
+def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor,
+                     block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
+                     pooled: Optional[torch.Tensor], B: int, max_new: int, nq: int, nkv: int, dk: int, dv: int, page: int,
+                     size: int, pool: int, scale: float, sink: bool) -> None:
+    """Steps of several tokens per sequence on the matrix cores: the same sums as `pwa_attend`, bfloat16 operands,
+    float scores and softmax, the weights rounded to bfloat16 for the second product."""
+    _dev("pwa_prefill_bf16", q, out, cu_seqlens, slots, ctx_lens, block_table, unit, pooled_table, pooled)
+    T = q.shape[0]
+    _req(pwa_prefill_takes(q.dtype, dk, dv, page), "pwa_prefill_bf16: bfloat16, pages of 64, key widths in steps of 8 and value "
+         "widths in steps of 4 up to 256")
+    _req(q.shape == (T, nq * dk) and out.shape == (T, nq * dv) and out.dtype == unit.dtype == torch.bfloat16,
+         "pwa_prefill_bf16: q [T, nq*dk], out [T, nq*dv], bfloat16 like the cache")
+    _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B and ctx_lens.numel() >= B, "pwa_prefill_bf16: arrays shorter than the batch")
+    _pwa_unit("pwa_prefill_bf16", unit, nkv, dk, dv, page)
+    if pool:
+        _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_prefill_bf16: pooled unit missing")
+        _pwa_unit("pwa_prefill_bf16", pooled, nkv, dk, dv, page)
+    f = _fn("pooled_attention", "br_pwa_prefill_bf16",
+            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P])
+    _check(f(_ptr(q), _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit),
+             _ptr(pooled_table), pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, max_new, nq, nkv, dk, dv,
+             int(size), int(pool), float(scale), int(sink), _stream()), "pwa_prefill_bf16")
+
+
 # ------------------------------------------------------ gated linear recurrence -----
-def glr_gates(rows: torch.Tensor, f_bias: Optional[torch.Tensor], lower: Optional[torch.Tensor], hd: int) -> None:
-    """rows [T, 2*hd + .] float: the first hd columns become silu(.), the next hd the forget gate
-    lower + (1 - lower) * sigmoid(. + f_bias)."""
-    _dev("glr_gates", rows, f_bias, lower)
-    _req(rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape[1] >= 2 * hd, "glr_gates: rows float32 [T, >= 2*hd]")
-    for v in (f_bias, lower):
-        _req(v is None or (v.dtype == torch.float32 and v.numel() == hd), "glr_gates: bias and lower bound float32 [hd]")
-    f = _fn("gated_recurrence", "br_glr_gates", [_P, _P, _P, c_int, c_int, c_int, _P])
-    _check(f(_ptr(rows), _ptr(f_bias), _ptr(lower), rows.shape[0], hd, rows.shape[1], _stream()), "glr_gates")
+def glr_rows_per_lane(d: int) -> int:
+    """Rows of a head's state that one lane of `glr_scan` holds: ceil(d / 16) rounded up to 4, 8, 16 or 32
+    (the kernel's own rule, `glr_rpl`; the launcher checks the state's size against it)."""
+    r = (int(d) + 15) // 16
+    return 4 if r <= 4 else (8 if r <= 8 else (16 if r <= 16 else 32))
 
 
-def glr_scan(rows: torch.Tensor, out: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor,
-             B: int, H: int, d: int, e: int) -> None:
-    """rows [T, 2*H*d + H*e] float (q | f | v, gates applied), state [slots, H, d, e] float: walks every
-    sequence's new tokens in order, writes o [T, H*e] float and leaves the state."""
-    _dev("glr_scan", rows, out, cu_seqlens, slots)
+def glr_state_shape(H: int, d: int, e: int):
+    """A sequence's recurrent state as `glr_scan` keeps it, [H, ceil(e/4), rows per lane, 64]: S[h][r][c] lies in
+    column block c // 4 at k = r % rows per lane, lane = 16 (c % 4) + r // rows per lane."""
+    return (H, (e + 3) // 4, glr_rows_per_lane(d), 64)
+
+
+def glr_state_dense(state: torch.Tensor, H: int, d: int, e: int) -> torch.Tensor:
+    """One slot's state [H, ceil(e/4), rows per lane, 64] as the plain S [H, d, e] (for tests and inspection)."""
+    ncb, rpl = (e + 3) // 4, glr_rows_per_lane(d)
+    t = state.reshape(H, ncb, rpl, 4, 16)                  # [h, cb, k, cg, g]
+    t = t.permute(0, 4, 2, 1, 3).reshape(H, 16 * rpl, ncb * 4)      # rows r = g * rpl + k, columns c = cb * 4 + cg
+    return t[:, :d, :e]
+
+
+def glr_scan(rows: torch.Tensor, f_bias: Optional[torch.Tensor], lower: Optional[torch.Tensor], out: torch.Tensor,
+             state: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, B: int, H: int, d: int, e: int) -> None:
+    """rows [T, 2*H*d + H*e] float, the projections' sums q | f | v; q = silu(.), f = lower + (1 - lower) *
+    sigmoid(. + f_bias) are applied on the way.  state [slots, *glr_state_shape]: walks every sequence's new
+    tokens in order, writes o [T, H*e] float and leaves the state."""
+    _dev("glr_scan", rows, f_bias, lower, out, cu_seqlens, slots)
     T = rows.shape[0]
-    _req(state.is_cuda and state.dim() == 4 and state[0].is_contiguous() and state.stride(0) >= H * d * e,
-         "glr_scan: every slot's state must be dense")
+    _req(state.is_cuda and state.shape[1:] == glr_state_shape(H, d, e) and state[0].is_contiguous(),
+         "glr_scan: state [slots, H, ceil(e/4), rows per lane, 64], every slot's dense")
     _req(rows.dtype == out.dtype == state.dtype == torch.float32, "glr_scan: float32 only")
     _req(rows.shape == (T, 2 * H * d + H * e) and out.shape == (T, H * e), "glr_scan: rows [T, 2*H*d + H*e], out [T, H*e]")
-    _req(state.dim() == 4 and state.shape[1:] == (H, d, e), "glr_scan: state [slots, H, d, e]")
+    for v in (f_bias, lower):
+        _req(v is None or (v.dtype == torch.float32 and v.numel() == H * d), "glr_scan: bias and lower bound float32 [H*d]")
     _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "glr_scan: arrays shorter than the batch")
     _req(d <= 512, f"glr_scan: {d} query channels a head are beyond the kernel's 512")
-    f = _fn("gated_recurrence", "br_glr_scan", [_P, _P, _P, _P, _P] + [c_int] * 5 + [c_size_t, _P])
-    _check(f(_ptr(rows), _ptr(out), _ptr(state), _ptr(cu_seqlens), _ptr(slots), B, H, d, e, rows.shape[1],
-             state.stride(0), _stream()), "glr_scan")
+    f = _fn("gated_recurrence", "br_glr_scan", [_P, _P, _P, _P, _P, _P, _P] + [c_int] * 5 + [c_size_t, _P])
+    _check(f(_ptr(rows), _ptr(f_bias), _ptr(lower), _ptr(out), _ptr(state), _ptr(cu_seqlens), _ptr(slots), B, H, d, e,
+             rows.shape[1], state.stride(0), _stream()), "glr_scan")
+
+
+def glr_scan_pieces(rows: torch.Tensor, f_bias: Optional[torch.Tensor], lower: Optional[torch.Tensor], out: torch.Tensor,
+                    state: torch.Tensor, slots: torch.Tensor, piece_cu: torch.Tensor, piece_slots: torch.Tensor,
+                    piece_state: torch.Tensor, decay: torch.Tensor, B: int, pieces: int, H: int, d: int, e: int) -> None:
+    """`glr_scan` of a step of long prompts with every sequence cut into `pieces` pieces that are walked side by
+    side (twice: from a zero state, then from their true first states).  `piece_cu` int32 [B*pieces + 1] cuts the
+    packed tokens, `piece_slots` int32 [B*pieces] numbers the pieces (-1: a padding sequence's); `piece_state`
+    float [B*pieces, *glr_state_shape] and `decay` float [B*pieces, H, 16 * rows per lane] are scratch."""
+    _dev("glr_scan_pieces", rows, f_bias, lower, out, slots, piece_cu, piece_slots, piece_state, decay)
+    T = rows.shape[0]
+    shape = glr_state_shape(H, d, e)
+    _req(state.is_cuda and state.shape[1:] == shape and state[0].is_contiguous(), "glr_scan_pieces: state [slots, *glr_state_shape]")
+    _req(rows.dtype == out.dtype == state.dtype == piece_state.dtype == decay.dtype == torch.float32, "glr_scan_pieces: float32 only")
+    _req(rows.shape == (T, 2 * H * d + H * e) and out.shape == (T, H * e), "glr_scan_pieces: rows [T, 2*H*d + H*e], out [T, H*e]")
+    _req(piece_state.shape == (B * pieces,) + tuple(shape) and decay.shape == (B * pieces, H, 16 * glr_rows_per_lane(d)),
+         "glr_scan_pieces: scratch of the wrong size")
+    _req(piece_cu.dtype == piece_slots.dtype == torch.int32 and piece_cu.numel() == B * pieces + 1 and piece_slots.numel() == B * pieces
+         and slots.numel() >= B, "glr_scan_pieces: piece arrays int32 [B*pieces + 1] and [B*pieces]")
+    for v in (f_bias, lower):
+        _req(v is None or (v.dtype == torch.float32 and v.numel() == H * d), "glr_scan_pieces: bias and lower bound float32 [H*d]")
+    f = _fn("gated_recurrence", "br_glr_scan_pieces", [_P] * 10 + [c_int] * 6 + [c_size_t, _P])
+    _check(f(_ptr(rows), _ptr(f_bias), _ptr(lower), _ptr(out), _ptr(state), _ptr(slots), _ptr(piece_cu), _ptr(piece_slots),
+             _ptr(piece_state), _ptr(decay), B, pieces, H, d, e, rows.shape[1], state.stride(0), _stream()), "glr_scan_pieces")
 
 
 def head_rmsnorm(o: torch.Tensor, w: Optional[torch.Tensor], out: torch.Tensor, H: int, e: int, eps: float) -> None:

@@ -87,10 +87,17 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
-    def add_normed(self, y: torch.Tensor, x: torch.Tensor) -> None:
+    def add_normed(self, y: torch.Tensor, x: torch.Tensor, then: Optional["Norm"] = None,
+                   then_out: Optional[torch.Tensor] = None) -> bool:
         """x += norm(y), both float [T, H]: the sum of a branch whose output is normed before it
-        joins the residual rows.  Norms without a kernel for it norm into a buffer and add."""
+        joins the residual rows.  With `then` (the norm that reads x next) and `then_out`, the norm may
+        also leave then_out = then(x) in the same kernel; it returns whether it did."""
         raise NotImplementedError
+
+    def then_args(self):
+        """(weight, eps, centered) for a norm kernel that applies this norm behind another one, or None
+        when the norm is not of that family."""
+        return None
 
     def prepare_in_product(self, a: torch.Tensor, w: torch.Tensor, x: torch.Tensor, ws) -> Any:
         """x += a @ w^T with this norm of the new x prepared in the same kernel, if the norm

@@ -32,6 +32,8 @@ def run_residual_branch(part, norm, next_norm, x, step, dtype, *extra) -> None:
     h = x
     if norm is not None:
         mine = prepared[2] if prepared is not None and prepared[0] is norm and prepared[1] is x else None
+        if isinstance(mine, tuple) and mine[:1] == ("normed",):
+            mine = None            # rows another arrangement normed ahead: not a product's preparation; norm again
         h = NormedInput(x, norm, step.ws, dtype, mine)
     sink = ResidualSink(x, next_norm)
     part.forward(h, sink, step, *extra)
@@ -62,26 +64,37 @@ class SandwichResidual:
     of each half and one behind it, before the sum.  Roles of `layer.norms`: "mixer", "mixer_out",
     "feed_forward", "feed_forward_out" (an absent one is left out).  The half writes its output
     into float rows of its own; the norm behind it adds the normed rows to the residual rows, so
-    the sum is a float add in that kernel."""
+    the sum is a float add in that kernel, and where it can it also leaves the norm that reads the
+    rows next (the other half's, or the next layer's first) in the same pass."""
+
+    def first_norm(self, layer):
+        return layer.norms.get("mixer") if layer.mixer is not None else layer.norms.get("feed_forward")
 
     def run(self, layer, x, step, mixer_ctx) -> None:
-        step.prepared_norm = None
+        after = step.norm_after_layer          # the norm that reads x after this layer, if known
+        ffn_norm = layer.norms.get("feed_forward")
         if layer.mixer is not None:
-            self.branch(layer.mixer, layer.norms.get("mixer"), layer.norms.get("mixer_out"), x, step, layer.rt.dtype, mixer_ctx)
+            nxt = ffn_norm if layer.feed_forward is not None else after
+            self.branch(layer.mixer, layer.norms.get("mixer"), layer.norms.get("mixer_out"), nxt, x, step, layer.rt.dtype, mixer_ctx)
         if step.probe is not None:
             step.probe(f"L{step.schedule_index}.post_mixer", x)
         if layer.feed_forward is not None:
-            self.branch(layer.feed_forward, layer.norms.get("feed_forward"), layer.norms.get("feed_forward_out"), x, step,
-                        layer.rt.dtype)
+            self.branch(layer.feed_forward, ffn_norm, layer.norms.get("feed_forward_out"), after, x, step, layer.rt.dtype)
         if step.probe is not None:
             step.probe(f"L{step.schedule_index}.post_ffn", x)
 
     @staticmethod
-    def branch(part, norm_in, norm_out, x, step, dtype, *extra) -> None:
+    def branch(part, norm_in, norm_out, next_norm, x, step, dtype, *extra) -> None:
+        prepared, step.prepared_norm = step.prepared_norm, None
         h = x
         if norm_in is not None:
-            h = step.ws.get("block_h", tuple(x.shape), dtype)
-            norm_in.forward(x, h)
+            # two buffers in turn: the norm behind this half writes the next half's input while this one's is read
+            if isinstance(prepared, tuple) and len(prepared) == 3 and prepared[0] is norm_in and prepared[1] is x \
+                    and isinstance(prepared[2], tuple) and prepared[2][0] == "normed":
+                h = prepared[2][1]
+            else:
+                h = step.ws.get("block_h", tuple(x.shape), dtype)
+                norm_in.forward(x, h)
         if norm_out is None:
             part.forward(h, x, step, *extra)
             return
@@ -91,7 +104,12 @@ class SandwichResidual:
         else:
             y.zero_()
             part.forward(h, y, step, *extra)
-        norm_out.add_normed(y, x)
+        h_next = None
+        if next_norm is not None and next_norm.then_args() is not None:
+            name = "block_h2" if h is not x and h.data_ptr() == step.ws.get("block_h", tuple(x.shape), dtype).data_ptr() else "block_h"
+            h_next = step.ws.get(name, tuple(x.shape), dtype)
+        if norm_out.add_normed(y, x, next_norm if h_next is not None else None, h_next):
+            step.prepared_norm = (next_norm, x, ("normed", h_next))
 
 
 register_part("block", "prenorm_residual", PrenormResidual, replace=True)

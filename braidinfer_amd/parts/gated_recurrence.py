@@ -8,9 +8,11 @@ head's o is RMS-normed over its e channels with one weight shared by the heads, 
 concatenated and projected by W_o.
 
 The state S [heads, d, e] starts at zero, lives in float in both precisions and is carried from
-step to step in the sequence's slot of the cache's state area (`StateNeed`); gates, the
-recurrence and the head norm are float.  Prompts are walked token by token inside one kernel,
-the state in registers.  The reference has no recurrent mixer of this form.
+step to step in the sequence's slot of the cache's state area (`StateNeed`, laid out as the scan
+kernel's lanes hold it); the gates' activations, the recurrence and the head norm are float.
+Prompts are walked token by token inside one kernel, a workgroup per 16 columns of a head's state
+with the state in registers and the tokens' rows staged through LDS a chunk ahead; long prompts that
+would leave the chip idle are cut into pieces that are walked side by side (`pieces_for`).  The reference has no recurrent mixer of this form.
 """
 from __future__ import annotations
 
@@ -63,7 +65,37 @@ class HGRN2(Mixer):
         self.norm_w = rt.own(tensors[prefix + n["norm"]].to(torch.float32))
 
     def state_need(self) -> StateNeed:
-        return StateNeed((self.nh, self.d, self.e), torch.float32)
+        return StateNeed(K.glr_state_shape(self.nh, self.d, self.e), torch.float32)
+
+    MIN_PIECE = 128          # tokens: shorter pieces do not pay for the second walk
+
+    def pieces_for(self, step) -> int:
+        """Into how many pieces a step's sequences are cut so that the walk fills the chip: a workgroup walks 16
+        columns of a head's state for one sequence, and a lone prompt of a small model has a few dozen of them.
+        One piece (the plain walk) for single tokens, short steps and batches that fill the chip already."""
+        if step.is_decode or step.max_new < 4 * self.MIN_PIECE:
+            return 1
+        units = step.n_seqs * self.nh * -(-self.e // 16)
+        want = (2 * K.device_cus()) // max(1, units)
+        return max(1, min(want, step.max_new // self.MIN_PIECE, 16, 65535 // max(1, step.n_seqs)))
+
+    @staticmethod
+    def _piece_arrays(step, pieces: int):
+        """(cuts of the packed tokens [B * pieces + 1], piece numbers [B * pieces]) on the device, made once per step
+        and number of pieces: sequence b's tokens in `pieces` runs of equal length (a multiple of 16), the last ones
+        shorter or empty."""
+        key = ("glr_pieces", pieces)
+        if key not in step.extras:
+            cu, numbers, at = [0], [], 0
+            for b, n in enumerate(step.host_new):
+                run = -(-(-(-n // pieces)) // 16) * 16
+                for c in range(pieces):
+                    cu.append(at + min(n, (c + 1) * run))
+                    numbers.append(b * pieces + c if step.host_slots[b] >= 0 else -1)
+                at += n
+            dev = torch.tensor(cu + numbers, dtype=torch.int32).to(step.tokens.device)
+            step.extras[key] = (dev[:len(cu)], dev[len(cu):])
+        return step.extras[key]
 
     def forward(self, h, x, step, ctx: MixerContext) -> None:
         T, nh, d, e = step.n_tokens, self.nh, self.d, self.e
@@ -72,9 +104,17 @@ class HGRN2(Mixer):
         # float sums of the three projections: the gates and the recurrence work on them unrounded
         rows = step.ws.get("glr_qfv", (T, 2 * nh * d + nh * e), torch.float32)
         linear(h, self.w_qfv, rows, step.ws)
-        K.glr_gates(rows, self.f_bias, self.lower, nh * d)
         o = step.ws.get("glr_o", (T, nh * e), torch.float32)
-        K.glr_scan(rows, o, ctx.state, step.cu_seqlens, step.slots, step.n_seqs, nh, d, e)
+        pieces = self.pieces_for(step)
+        if pieces > 1:
+            cu, numbers = self._piece_arrays(step, pieces)
+            n = step.n_seqs * pieces
+            piece_state = step.ws.get("glr_piece_state", (n,) + tuple(K.glr_state_shape(nh, d, e)), torch.float32)
+            decay = step.ws.get("glr_decay", (n, nh, 16 * K.glr_rows_per_lane(d)), torch.float32)
+            K.glr_scan_pieces(rows, self.f_bias, self.lower, o, ctx.state, step.slots, cu, numbers, piece_state, decay,
+                              step.n_seqs, pieces, nh, d, e)
+        else:
+            K.glr_scan(rows, self.f_bias, self.lower, o, ctx.state, step.cu_seqlens, step.slots, step.n_seqs, nh, d, e)
         on = step.ws.get("glr_on", (T, nh * e), self.rt.dtype)
         K.head_rmsnorm(o, self.norm_w, on, nh, e, self.eps)
         linear(on, self.w_o, x, step.ws, accumulate=True)

@@ -35,8 +35,14 @@ class RMSNorm(Norm):
         K.rmsnorm(x, self.weight, out, self.eps, rows)
         return out
 
-    def add_normed(self, y, x):
-        K.layernorm(y, self.weight, x, self.eps, center=False, add=True)
+    def then_args(self):
+        return self.weight, self.eps, False
+
+    def add_normed(self, y, x, then=None, then_out=None):
+        nxt = then.then_args() if then is not None and then_out is not None else None
+        K.layernorm(y, self.weight, x, self.eps, center=False, add=True,
+                    then=(nxt[0], then_out, nxt[1], nxt[2]) if nxt else None)
+        return nxt is not None
 
     def prepare_in_product(self, a, w, x, ws):
         M, N = x.shape
@@ -88,8 +94,14 @@ class LayerNorm(Norm):
         K.layernorm(x, self.weight, out, self.eps, rows, center=True)
         return out
 
-    def add_normed(self, y, x):
-        K.layernorm(y, self.weight, x, self.eps, center=True, add=True)
+    def then_args(self):
+        return self.weight, self.eps, True
+
+    def add_normed(self, y, x, then=None, then_out=None):
+        nxt = then.then_args() if then is not None and then_out is not None else None
+        K.layernorm(y, self.weight, x, self.eps, center=True, add=True,
+                    then=(nxt[0], then_out, nxt[1], nxt[2]) if nxt else None)
+        return nxt is not None
 
 
 register_part("norm", "rmsnorm", RMSNorm, replace=True)

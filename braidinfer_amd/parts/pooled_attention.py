@@ -82,6 +82,7 @@ class PooledWindowAttention(Mixer):
         self.names = dict(self.NAMES, **(names or {}))
         self.w_qkv = self.w_o = self.b_qkv = self.q_norm = self.k_norm = self.mix = None
         self._expects_tables = False
+        self.force_simple = False          # tests set it to run the one-wave-per-query kernel in bfloat16
 
     # ---- weights -----------------------------------------------------------------------
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
@@ -177,9 +178,17 @@ class PooledWindowAttention(Mixer):
             K.pwa_pool(unit, ctx.block_table, pooled.storage, pooled.block_table, step.cu_seqlens, step.ctx_lens, step.slots,
                        step.n_seqs, step.max_new, nkv, dk, dv, ctx.page_tokens, self.pool)
         o = step.ws.get("pwa_out", (T, nq * dv), dt)
-        K.pwa_attend(q, o, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit,
-                     pooled.block_table if pooled is not None else None, pooled.storage if pooled is not None else None,
-                     nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
+        p_table = pooled.block_table if pooled is not None else None
+        p_unit = pooled.storage if pooled is not None else None
+        if not step.is_decode and not self.force_simple and K.pwa_prefill_takes(dt, dk, dv, ctx.page_tokens):
+            # prompts and portions in bfloat16: the matrix cores
+            K.pwa_prefill_bf16(q, o, step.cu_seqlens, step.slots, step.ctx_lens, ctx.block_table, unit, p_table, p_unit,
+                               step.n_seqs, step.max_new, nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool,
+                               self.scale, self.sink)
+        else:
+            # single tokens, the 32-bit path and other sizes: one wave per (query, head) in float
+            K.pwa_attend(q, o, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit, p_table, p_unit,
+                         nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
 

@@ -58,7 +58,7 @@ def test_tensor_names_and_units():
     assert [n for n in names if n.startswith("l1.mix.")] == ["l1.mix." + x for x in ("q", "f", "f.b", "lower", "v", "norm", "o")]
     needs = model.cache_needs()
     assert sorted(needs) == [0, 3, 4, 7] and needs[4].tokens_per_row == 4 and needs[0].live_from is needs[3].live_from
-    assert {k: v.shape for k, v in model.state_needs().items()} == {("entry", 1): (3, 16, 32), ("entry", 2): (3, 16, 32)}
+    assert sorted(model.state_needs()) == [("entry", 1), ("entry", 2)]
 
 
 def test_which_token_rows_stay():

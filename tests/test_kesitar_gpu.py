@@ -132,7 +132,7 @@ def test_layer_norm_kernels():
 
 @pytest.mark.parametrize("H,d,e", [(2, 16, 32), (1, 18, 80), (3, 6, 8), (2, 128, 128), (1, 70, 200)])
 def test_gated_recurrence_kernels(H, d, e):
-    """gates, scan and head norm against the plain recurrence: two sequences in unequal portions, the state
+    """scan (with its gates) and head norm against the plain recurrence: two sequences in unequal portions, the state
     carried in slots that are not neighbours, a padding sequence between them."""
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(d)
@@ -148,8 +148,10 @@ def test_gated_recurrence_kernels(H, d, e):
         f = (lower + (1 - lower) * P.sigmoid(r[:, H * d:2 * H * d] + bias)).reshape(-1, H, d)
         o, S = P.gated_recurrence(q, f, r[:, 2 * H * d:].reshape(-1, H, e))
         want.append((P.rms_norm(o, nw, 1e-5).reshape(-1, H * e), S))
-    arena = torch.zeros((6, H * d * e + 8), dtype=torch.float32, device="cuda")      # slots with a gap between them
-    state = arena[:, 4:4 + H * d * e].view(6, H, d, e)
+    shape = K.glr_state_shape(H, d, e)                   # the state lies as the kernel's lanes hold it
+    n_state = int(np.prod(shape))
+    arena = torch.zeros((6, n_state + 8), dtype=torch.float32, device="cuda")      # slots with a gap between them
+    state = arena[:, 4:4 + n_state].view(6, *shape)
     slots_of = [4, 1]
     got = [[], []]
     for portion in ([20, 3], [1, 1], [16, 1]):
@@ -159,9 +161,8 @@ def test_gated_recurrence_kernels(H, d, e):
         rows = torch.tensor(np.concatenate(pieces)).cuda()
         cu = torch.tensor(np.cumsum([0, portion[0], 1, portion[1]]), dtype=torch.int32).cuda()
         slots = torch.tensor([slots_of[0], -1, slots_of[1]], dtype=torch.int32).cuda()
-        K.glr_gates(rows, torch.tensor(bias).cuda(), torch.tensor(lower).cuda(), H * d)
         o = torch.zeros((rows.shape[0], H * e), dtype=torch.float32, device="cuda")
-        K.glr_scan(rows, o, state, cu, slots, 3, H, d, e)
+        K.glr_scan(rows, torch.tensor(bias).cuda(), torch.tensor(lower).cuda(), o, state, cu, slots, 3, H, d, e)
         on = torch.empty_like(o)
         K.head_rmsnorm(o, torch.tensor(nw).cuda(), on, H, e, 1e-5)
         on = on.cpu().numpy()
@@ -170,9 +171,57 @@ def test_gated_recurrence_kernels(H, d, e):
     for i in range(2):
         g = np.concatenate(got[i])
         assert np.abs(g - want[i][0][:len(g)]).max() < 3e-4 * max(1.0, np.abs(want[i][0]).max())
-    full = state[slots_of[1]].cpu().numpy()            # the second sequence was run to its end
+    full = K.glr_state_dense(state[slots_of[1]], H, d, e).cpu().numpy()      # the second sequence ran to its end
     assert np.abs(full - want[1][1]).max() < 1e-4 * max(1.0, np.abs(want[1][1]).max())
     assert float(arena[:, :4].abs().max()) == 0 and float(arena[[0, 2, 3, 5]].abs().max()) == 0
+
+
+@pytest.mark.parametrize("H,d,e,pieces", [(2, 16, 32, 3), (1, 18, 80, 5), (2, 128, 128, 4), (1, 70, 200, 2)])
+def test_recurrence_in_pieces(H, d, e, pieces):
+    """Long prompts cut into pieces that are walked side by side, against the plain recurrence: from a state that is
+    not zero, with a padding sequence, a sequence shorter than the number of pieces and one whose last pieces are empty."""
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(e)
+    lens = [150, 3, 33]
+    raw = [rng.standard_normal((n + 20, 2 * H * d + H * e)).astype(np.float32) * 2 for n in lens]
+    bias = rng.standard_normal(H * d).astype(np.float32)
+    lower = rng.uniform(0.05, 0.9, H * d).astype(np.float32)
+    shape = K.glr_state_shape(H, d, e)
+    state = torch.zeros((5,) + tuple(shape), dtype=torch.float32, device="cuda")
+    slots_of = [3, 0, 4]
+    dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32).cuda()
+    bd, ld = torch.tensor(bias).cuda(), torch.tensor(lower).cuda()
+    # the first 20 tokens of each by the plain walk, so that the pieces start from a state
+    first = torch.tensor(np.concatenate([r[:20] for r in raw])).cuda()
+    o0 = torch.zeros((60, H * e), dtype=torch.float32, device="cuda")
+    K.glr_scan(first, bd, ld, o0, state, dev([0, 20, 40, 60]), dev(slots_of), 3, H, d, e)
+    rest = [r[20:] for r in raw]
+    pad = np.zeros((1, raw[0].shape[1]), np.float32)
+    rows = torch.tensor(np.concatenate([rest[0], pad, rest[1], rest[2]])).cuda()
+    new = [lens[0], 1, lens[1], lens[2]]
+    slots = [slots_of[0], -1, slots_of[1], slots_of[2]]
+    cu, numbers, at = [0], [], 0
+    for b, n in enumerate(new):
+        run = -(-(-(-n // pieces)) // 16) * 16
+        for c in range(pieces):
+            cu.append(at + min(n, (c + 1) * run))
+            numbers.append(b * pieces + c if slots[b] >= 0 else -1)
+        at += n
+    o = torch.zeros((rows.shape[0], H * e), dtype=torch.float32, device="cuda")
+    piece_state = torch.full((4 * pieces,) + tuple(shape), 7.0, dtype=torch.float32, device="cuda")
+    decay = torch.full((4 * pieces, H, 16 * K.glr_rows_per_lane(d)), 7.0, dtype=torch.float32, device="cuda")
+    K.glr_scan_pieces(rows, bd, ld, o, state, dev(slots), dev(cu), dev(numbers), piece_state, decay, 4, pieces, H, d, e)
+    o = o.cpu().numpy()
+    offs = [0, lens[0] + 1, lens[0] + 1 + lens[1]]
+    for i, r in enumerate(raw):
+        r = r.astype(np.float64)
+        q = P.silu(r[:, :H * d]).reshape(-1, H, d)
+        f = (lower + (1 - lower) * P.sigmoid(r[:, H * d:2 * H * d] + bias)).reshape(-1, H, d)
+        want, S = P.gated_recurrence(q, f, r[:, 2 * H * d:].reshape(-1, H, e))
+        got = o[offs[i]:offs[i] + lens[i]]
+        assert np.abs(got - want[20:].reshape(lens[i], -1)).max() < 3e-4 * max(1.0, np.abs(want).max())
+        assert np.abs(K.glr_state_dense(state[slots_of[i]], H, d, e).cpu().numpy() - S).max() < 1e-4 * max(1.0, np.abs(S).max())
+    assert float(state[[1, 2]].abs().max()) == 0
 
 
 class HandCache:
@@ -189,8 +238,9 @@ class HandCache:
         self.pooled = torch.full((n_pages, G * 64 * (dk + dv)), 1e4, dtype=dtype, device="cuda")
 
 
-def attend_in_portions(q, k, v, size, pool, scale, sink, portions, dtype=torch.float32, slot=1):
-    """q [T, H, dk], k [T, G, dk], v [T, G, dv] through prepare (no bias, norm or rotation), pool and attend."""
+def attend_in_portions(q, k, v, size, pool, scale, sink, portions, dtype=torch.float32, slot=1, matrix=False):
+    """q [T, H, dk], k [T, G, dk], v [T, G, dv] through prepare (no bias, norm or rotation), pool and attend
+    (`matrix`: portions of more than one token through the matrix-core kernel)."""
     from braidinfer_amd import kernels as K
     T, H, dk = q.shape
     G, dv = k.shape[1], v.shape[2]
@@ -207,8 +257,12 @@ def attend_in_portions(q, k, v, size, pool, scale, sink, portions, dtype=torch.f
         if pool:
             K.pwa_pool(c.unit, c.table, c.pooled, c.ptable, cu, ctx, slots, 2, n, G, dk, dv, 64, pool)
         o = torch.empty((n, H * dv), dtype=dtype, device="cuda")
-        K.pwa_attend(qo, o, pos, sot, slots, c.table, c.unit, c.ptable if pool else None, c.pooled if pool else None, H, G, dk, dv,
-                     64, size, pool, scale, sink)
+        if matrix and n > 1:
+            K.pwa_prefill_bf16(qo, o, cu, slots, ctx, c.table, c.unit, c.ptable if pool else None, c.pooled if pool else None, 2, n,
+                               H, G, dk, dv, 64, size, pool, scale, sink)
+        else:
+            K.pwa_attend(qo, o, pos, sot, slots, c.table, c.unit, c.ptable if pool else None, c.pooled if pool else None, H, G, dk,
+                         dv, 64, size, pool, scale, sink)
         outs.append(o.float().cpu().numpy())
         at += n
     return np.concatenate(outs).reshape(T, H, dv)
@@ -232,6 +286,13 @@ def test_pooled_window_attention_kernels(H, G, dk, dv, size, pool):
     # pooled rows are rounded to bfloat16 where they are kept, and so is the output
     want = P.pooled_window_attention(P.to_bf16(q), kb, vb, 0.4, size, pool, True)
     assert np.abs(got - want).max() < 0.03 * np.abs(want).max()
+    for sink in (True, False):
+        # the matrix-core kernel against the float one on the same cache: whole, and in portions whose edges
+        # fall inside a block of 32 keys, at a page's border and just behind it
+        plain = attend_in_portions(P.to_bf16(q), kb, vb, size, pool, 0.4, sink, [T], dtype=torch.bfloat16)
+        for portions in ([T], [33, 31, 2, 63, 65, 100, 6], [129, 171]):
+            fast = attend_in_portions(P.to_bf16(q), kb, vb, size, pool, 0.4, sink, portions, dtype=torch.bfloat16, matrix=True)
+            assert np.abs(fast - plain).max() < 0.03 * np.abs(plain).max()
 
 
 def test_edges_that_random_inputs_would_hide():
@@ -250,6 +311,8 @@ def test_edges_that_random_inputs_would_hide():
         want = P.pooled_window_attention(q, k, v, 1.0, size, pool, True)
         got = attend_in_portions(q, k, v, size, pool, 1.0, True, [T - 30] + [1] * 30)
         assert np.abs(got - want).max() < 2e-5
+        fast = attend_in_portions(q, P.to_bf16(k), P.to_bf16(v), size, pool, 1.0, True, [T - 40, 40], dtype=torch.bfloat16, matrix=True)
+        assert np.abs(fast - P.pooled_window_attention(q, P.to_bf16(k), P.to_bf16(v), 1.0, size, pool, True)).max() < 0.03
         i = T - 1
         inside = i - loud < size
         blk = loud // pool
@@ -307,7 +370,7 @@ def test_prepare_norm_rotation_and_value_mix():
         for p in pos:
             page = unit[table[1, p // 64]]
             ks.append(page[:G * 64 * dk].reshape(G, 64, dk)[:, p % 64])
-            vs.append(page[G * 64 * dk:].reshape(G, 64, dv)[:, p % 64])
+            vs.append(page[G * 64 * dk:].reshape(G, dv, 64)[:, :, p % 64])      # values lie transposed in a page
         return np.stack(ks), np.stack(vs).reshape(T, -1)
     ck, cv = cached()
     assert np.abs(ck - k).max() < 4e-4 and np.abs(cv - v).max() < 1e-6
@@ -418,6 +481,19 @@ def test_greedy_generation_through_the_engine(folders, engines):
                 l = P.forward(cfg, w, p + wnt[:i])[-1]
                 assert abs(l[a] - l[b]) < 0.05 * np.abs(l).max()
                 break
+
+
+def test_a_long_prompt_in_pieces(folders, engines):
+    """A prompt long enough for the recurrent layers to walk it in pieces, whole and behind a first portion."""
+    _, cfg, w = folders["a"]
+    toks = tokens_of(cfg, 700, 8)
+    want = P.forward(cfg, w, toks)
+    for dtype in ("float32", "bfloat16"):
+        eng = engines("a", dtype)
+        hg = [l.mixer for l in eng.model.layers if type(l.mixer).__name__ == "HGRN2"]
+        assert hg and all(m.MIN_PIECE * 4 <= 600 for m in hg)
+        close(run(eng, toks, [700]), want, dtype, f"whole {dtype}")
+        close(run(eng, toks, [100, 600]), want, dtype, f"behind a portion {dtype}")
 
 
 def test_presets_run(tmp_path):
