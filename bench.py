@@ -71,7 +71,7 @@ def measured_peaks(torch, K):
 
 LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_kv_write", "silu_mul", "residual_add", "gather_rows",
              "convert", "gemm", "gemm_swiglu", "gemm_norm_prepare", "gemm_norm_scaled", "attention_simple",
-             "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16",
+             "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16", "pwa_decode_bf16",
              "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax"]
 
 

@@ -521,6 +521,158 @@ __global__ __launch_bounds__(256) void pwa_prefill_kernel(
         }
 }
 
+// ------------------------------------------------ single tokens on the matrix cores -----
+// Steps of one token per sequence, bfloat16: grid = (nkv, sequences), block = 256.  The G query heads of a kv
+// head are the columns of the score blocks (G <= 32; the other columns idle), so the keys and values of a kv
+// head are read once for all of its query heads.  The blocks of 32 keys the token sees (pooled rows first,
+// then its window) are dealt to the four waves in turn; each wave runs the online softmax over its blocks
+// (wave 0 starts with the sink), and the four (m, l, O) are merged through LDS in wave order.
+template <int NBK, int NBV>
+__global__ __launch_bounds__(256) void pwa_decode_kernel(
+    const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ slots,
+    const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
+    const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+    extern __shared__ float lds[];
+    const int b = blockIdx.y, kvh = blockIdx.x;
+    const int slot = slots[b];
+    const int G = nq / nkv;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, g = lane >> 5;
+    const bool row_ok = c < G;
+    const int head = kvh * G + (row_ok ? c : G - 1);
+    if (slot < 0) {       // padding: no cache behind it
+        for (int i = threadIdx.x; i < G * dv; i += 256) out[((size_t)b * nq + kvh * G) * dv + i] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], pq = ctx - 1;
+    const bf16* qrow = q + ((size_t)b * nq + head) * dk;
+    bf16x8 qf[2 * NBK];
+#pragma unroll
+    for (int s = 0; s < 2 * NBK; ++s) {
+        const int d = s * 16 + 8 * g;
+        qf[s] = (d < dk) ? *(const bf16x8*)(qrow + d) : pwa_zero8();
+    }
+    f32x16 acc_o[NBV];
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    float m = (sink && wave == 0) ? 0.f : -INFINITY, lsum = (sink && wave == 0 && g == 0) ? 1.f : 0.f;
+    const float scale2 = scale * PWA_LOG2E;
+    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
+    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+    int seen = 0;
+    if (pool > 0 && pq - size - pool + 1 >= 0) seen = (pq - size - pool + 1) / pool + 1;
+    const int far_blocks = (seen + 31) / 32;
+    int lo = pq - size + 1;
+    if (lo < 0) lo = 0;
+    const int kb0 = (lo / 32) * 32;
+    const int n_blocks = far_blocks + (pq - kb0) / 32 + 1;
+    const int* bt = block_table + (size_t)slot * table_stride;
+    const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
+    for (int n = wave; n < n_blocks; n += 4) {
+        const bool far = n < far_blocks;
+        const int kb = far ? n * 32 : kb0 + (n - far_blocks) * 32;
+        const int kl = kb % PWA_PAGE;
+        const bf16* pg = far ? pooled + (size_t)pt[kb / PWA_PAGE] * page_elems : storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
+        const int limit = (far ? ctx / pool : ctx) - (kb - kl);
+        const int first_ok = row_ok ? (far ? 0 : lo) : 1, last_ok = row_ok ? (far ? seen - 1 : pq) : 0;
+        pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, limit, first_ok, last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    // merge: [wave][2 G lanes] of m and l, [wave][NBV * 16][2 G lanes] of O
+    const int nl = 2 * G, li = g * G + c;
+    float* mL = lds;                       // [4][nl]
+    float* lL = mL + 4 * nl;               // [4][nl]
+    float* oL = lL + 4 * nl;               // [4][NBV * 16][nl]
+    if (row_ok) {
+        mL[wave * nl + li] = m;
+        lL[wave * nl + li] = lsum;
+#pragma unroll
+        for (int i = 0; i < NBV; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oL[((size_t)wave * NBV * 16 + i * 16 + r) * nl + li] = acc_o[i][r];
+    }
+    __syncthreads();
+    if (wave != 0 || !row_ok) return;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, mL[w * nl + li]);
+    float cw[4], L = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const float mw = mL[w * nl + li];
+        cw[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+        L += lL[w * nl + li] * cw[w];
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+    bf16* orow = out + ((size_t)b * nq + head) * dv;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;
+            if (d < dv) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) a += oL[((size_t)w * NBV * 16 + i * 16 + 4 * r4 + e) * nl + li] * cw[w];
+                    o[e] = (bf16)(a * inv);
+                }
+                *(bf16x4*)(orow + d) = o;
+            }
+        }
+}
+
+template <int NBK>
+static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStream_t s, const bf16* q, bf16* out, const int* slots,
+                               const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
+                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, size_t head_lds) {
+#define PWA_GO(V) pwa_decode_kernel<NBK, V><<<grid, 256, head_lds + lds_of_nbv16 * V, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink)
+    if (nbv <= 1) PWA_GO(1);
+    else if (nbv <= 2) PWA_GO(2);
+    else if (nbv <= 3) PWA_GO(3);
+    else if (nbv <= 4) PWA_GO(4);
+    else PWA_GO(8);
+#undef PWA_GO
+    return br_check_launch();
+}
+
+// Bytes of LDS the merge of `pwa_decode_kernel` needs for these sizes (the launcher refuses more than 64 KB).
+static size_t pwa_decode_lds(int G, int dv) {
+    const int nbv = (dv + 31) / 32, v = nbv <= 4 ? nbv : 8;
+    return (size_t)(8 * 2 * G + 4 * v * 16 * 2 * G) * sizeof(float);
+}
+extern "C" int br_pwa_decode_takes(int nq, int nkv, int dk, int dv) {
+    if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 || dv % 4) return 0;
+    return pwa_decode_lds(nq / nkv, dv) <= 65536;
+}
+
+extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, const int* ctx_lens, const int* block_table,
+                                  int table_stride, const void* storage, const int* pooled_table, int pooled_stride,
+                                  const void* pooled, int B, int nq, int nkv, int dk, int dv, int size, int pool, float scale,
+                                  int sink, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (!br_pwa_decode_takes(nq, nkv, dk, dv) || nkv > 65535 || B > 65535 || size <= 0 || pool < 0 ||
+        (pool > 0 && (!pooled_table || !pooled)))
+        return BR_BAD_ARG;
+    const int G = nq / nkv;
+    dim3 grid(nkv, B);
+    const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
+    const size_t head_lds = (size_t)8 * 2 * G * sizeof(float), per_v = (size_t)4 * 16 * 2 * G * sizeof(float);
+#define PWA_K(KK) pwa_decode_launch_v<KK>(nbv, grid, per_v, s, (const bf16*)q, (bf16*)out, slots, ctx_lens, block_table, table_stride, \
+                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, head_lds)
+    if (nbk <= 1) return PWA_K(1);
+    if (nbk <= 2) return PWA_K(2);
+    if (nbk <= 3) return PWA_K(3);
+    if (nbk <= 4) return PWA_K(4);
+    return PWA_K(8);
+#undef PWA_K
+}
+
 template <int NBK>
 static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
                                 const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,

@@ -16,6 +16,7 @@ would leave the chip idle are cut into pieces that are walked side by side (`pie
 """
 from __future__ import annotations
 
+import os
 from typing import Dict, List, Optional
 
 import torch
@@ -75,8 +76,12 @@ class HGRN2(Mixer):
         One piece (the plain walk) for single tokens, short steps and batches that fill the chip already."""
         if step.is_decode or step.max_new < 4 * self.MIN_PIECE:
             return 1
+        # a workgroup is four waves, one to a SIMD, and a lone wave waits out every latency of its token loop, so
+        # pieces are asked for until four workgroups share a compute unit (BRAIDINFER_GLR_FILL, for measurements;
+        # a prompt of 8,192 tokens through 8 layers of width 2,048 / 4,096: 17.8 / 43.3 ms at 1, 13.7 / 40.2 at 2,
+        # 12.9 / 38.4 at 4, 12.8 / 38.1 at 8)
         units = step.n_seqs * self.nh * -(-self.e // 16)
-        want = (2 * K.device_cus()) // max(1, units)
+        want = (int(os.environ.get("BRAIDINFER_GLR_FILL", "4")) * K.device_cus()) // max(1, units)
         return max(1, min(want, step.max_new // self.MIN_PIECE, 16, 65535 // max(1, step.n_seqs)))
 
     @staticmethod

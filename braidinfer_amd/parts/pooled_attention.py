@@ -185,8 +185,12 @@ class PooledWindowAttention(Mixer):
             K.pwa_prefill_bf16(q, o, step.cu_seqlens, step.slots, step.ctx_lens, ctx.block_table, unit, p_table, p_unit,
                                step.n_seqs, step.max_new, nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool,
                                self.scale, self.sink)
+        elif step.is_decode and not self.force_simple and K.pwa_decode_takes(dt, nq, nkv, dk, dv, ctx.page_tokens):
+            # single tokens in bfloat16: the matrix cores, a kv head's keys read once for its query heads
+            K.pwa_decode_bf16(q, o, step.slots, step.ctx_lens, ctx.block_table, unit, p_table, p_unit, step.n_seqs,
+                              nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
         else:
-            # single tokens, the 32-bit path and other sizes: one wave per (query, head) in float
+            # the 32-bit path and other sizes: four waves per (query, head) in float
             K.pwa_attend(q, o, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit, p_table, p_unit,
                          nq, nkv, dk, dv, ctx.page_tokens, self.window, self.pool, self.scale, self.sink)
         linear(o, self.w_o, x, step.ws, accumulate=True)

@@ -257,7 +257,11 @@ def attend_in_portions(q, k, v, size, pool, scale, sink, portions, dtype=torch.f
         if pool:
             K.pwa_pool(c.unit, c.table, c.pooled, c.ptable, cu, ctx, slots, 2, n, G, dk, dv, 64, pool)
         o = torch.empty((n, H * dv), dtype=dtype, device="cuda")
-        if matrix and n > 1:
+        if matrix and n == 1:
+            K.pwa_decode_bf16(qo[:1].repeat(2, 1), o2 := torch.empty((2, H * dv), dtype=dtype, device="cuda"), slots, ctx, c.table,
+                              c.unit, c.ptable if pool else None, c.pooled if pool else None, 2, H, G, dk, dv, 64, size, pool, scale, sink)
+            o = o2[1:]                    # row b of a single-token step is sequence b: the first is padding
+        elif matrix:
             K.pwa_prefill_bf16(qo, o, cu, slots, ctx, c.table, c.unit, c.ptable if pool else None, c.pooled if pool else None, 2, n,
                                H, G, dk, dv, 64, size, pool, scale, sink)
         else:
@@ -290,7 +294,7 @@ def test_pooled_window_attention_kernels(H, G, dk, dv, size, pool):
         # the matrix-core kernel against the float one on the same cache: whole, and in portions whose edges
         # fall inside a block of 32 keys, at a page's border and just behind it
         plain = attend_in_portions(P.to_bf16(q), kb, vb, size, pool, 0.4, sink, [T], dtype=torch.bfloat16)
-        for portions in ([T], [33, 31, 2, 63, 65, 100, 6], [129, 171]):
+        for portions in ([T], [33, 31, 2, 63, 65, 100, 6], [129, 171], [T - 45] + [1] * 45):
             fast = attend_in_portions(P.to_bf16(q), kb, vb, size, pool, 0.4, sink, portions, dtype=torch.bfloat16, matrix=True)
             assert np.abs(fast - plain).max() < 0.03 * np.abs(plain).max()
 
