@@ -111,7 +111,9 @@ def main(argv=None) -> int:
         # and every live request may leave its last page partly empty, so the pages are counted generously
         longest = max(args.max_tokens, 64)
         room = 2 * longest + 64 * 64
-        engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device, max_tokens=room, max_seq_len=longest)
+        # a slot per live request: a model with recurrent layers keeps a state per slot, so slots are not counted by pages
+        engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device, max_tokens=room, max_seq_len=longest,
+                                    n_slots=min(-(-room // 64), 512))
         Replayer(engine, args.out, probes=args.probes).run(sys.stdin, sys.stdout)
     except BraidError as e:
         print(f"trace_run: {type(e).__name__}: {e}", file=sys.stderr, flush=True)

@@ -44,6 +44,10 @@ CONFIGS = {
     # windows and blocks longer than a page of 64 tokens
     "c": model(32, 64, [attention(2, 1, 16, 16, 70, 66, rot=(8, 1e4), v_mix=True, mlp=48), hgrn2(2, 8, 8),
                         attention(2, 1, 16, 16, 130, 5, rot=(8, 1e4), v_mix=True, mlp=48)]),
+    # recurrent layers first and last, the values' source in the middle of the stack, many query heads to a kv head,
+    # a width that is no multiple of 4, value channels that are no multiple of 4, odd query channels
+    "d": model(50, 131, [hgrn2(2, 9, 7, mlp=36), attention(8, 1, 8, 12, 11, 2, rot=(6, 300.0), v_mix=True, mlp=36),
+                         attention(2, 1, 12, 12, 4, 6, v_mix=True), hgrn2(1, 33, 16, mlp=20)], emb=2.0, out=0.5),
 }
 
 
