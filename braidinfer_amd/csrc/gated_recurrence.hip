@@ -282,23 +282,50 @@ extern "C" int br_glr_scan_pieces(const float* rows, const float* f_bias, const 
 }
 
 // ------------------------------------------------------------------ head norm ------
-// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w, one wave per (token, head).
-template <typename T>
-__global__ __launch_bounds__(64) void glr_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
-                                                           T* __restrict__ y, int e, float eps) {
-    const size_t base = ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * e;
+// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w.  16 lanes a (token, head) row, 16 rows a
+// workgroup: a row of 128 channels is two 16-byte loads a lane, its sum of squares four moves between
+// neighbouring lanes in a fixed order.
+template <typename T, bool V4>
+__global__ __launch_bounds__(256) void glr_head_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                            T* __restrict__ y, size_t n_rows, int e, float eps) {
+    const size_t r = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int l = threadIdx.x & 15;
+    const bool on = r < n_rows;
+    const float* orow = o + (on ? r : 0) * e;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < e; i += 64) { const float v = o[base + i]; ss += v * v; }
-    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)e + eps);
-    for (int i = threadIdx.x; i < e; i += 64) y[base + i] = from_f32<T>(o[base + i] * inv * (w ? w[i] : 1.0f));
+    if (V4) {
+        for (int i = l; i < (e >> 2); i += 16) {
+            const f32x4 v = on ? ((const f32x4*)orow)[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+            ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        }
+    } else {
+        for (int i = l; i < e; i += 16) { const float v = on ? orow[i] : 0.f; ss += v * v; }
+    }
+    const float inv = 1.0f / sqrtf(glr_row16_sum(ss) / (float)e + eps);
+    if (!on) return;
+    T* yrow = y + r * e;
+    if (V4) {
+        for (int i = l; i < (e >> 2); i += 16) {
+            const f32x4 v = ((const f32x4*)orow)[i];
+            const f32x4 wv = w ? ((const f32x4*)w)[i] : f32x4{1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+            for (int x = 0; x < 4; ++x) yrow[4 * i + x] = from_f32<T>(v[x] * inv * wv[x]);
+        }
+    } else {
+        for (int i = l; i < e; i += 16) yrow[i] = from_f32<T>(orow[i] * inv * (w ? w[i] : 1.0f));
+    }
 }
 
 extern "C" int br_glr_head_norm(const float* o, const float* w, void* y, int y_is_bf16, int T, int H, int e,
                                 float eps, hipStream_t s) {
     if (T <= 0) return BR_OK;
-    if (H <= 0 || H > 65535 || e <= 0) return BR_BAD_ARG;
-    dim3 grid(T, H);
-    if (y_is_bf16) glr_head_norm_kernel<bf16><<<grid, 64, 0, s>>>(o, w, (bf16*)y, e, eps);
-    else glr_head_norm_kernel<float><<<grid, 64, 0, s>>>(o, w, (float*)y, e, eps);
+    if (H <= 0 || e <= 0) return BR_BAD_ARG;
+    const size_t n_rows = (size_t)T * H;
+    const unsigned blocks = (unsigned)((n_rows + 15) / 16);
+    const bool v4 = e % 4 == 0 && (((uintptr_t)o | (uintptr_t)w) % 16) == 0;
+#define GLR_HN(TT, V) glr_head_norm_kernel<TT, V><<<blocks, 256, 0, s>>>(o, w, (TT*)y, n_rows, e, eps)
+    if (y_is_bf16) { if (v4) GLR_HN(bf16, true); else GLR_HN(bf16, false); }
+    else { if (v4) GLR_HN(float, true); else GLR_HN(float, false); }
+#undef GLR_HN
     return br_check_launch();
 }

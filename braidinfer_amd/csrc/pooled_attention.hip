@@ -66,7 +66,8 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
             ss += v[j] * v[j];
         }
     }
-    if (is_q || is_k) {
+    const bool qk = is_q || is_k;
+    if (qk) {
         const float* nw = is_q ? qn_w : kn_w;
         if (nw) {
             const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
@@ -76,14 +77,18 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
                 if (i < n) v[j] = v[j] * inv * nw[i];
             }
         }
-        if (rd > 0) {
-            const int half = rd >> 1;
+    }
+    if (rd > 0) {                           // the barrier is met whatever the head
+        const int half = rd >> 1;
+        if (qk) {
 #pragma unroll
             for (int j = 0; j < MAX_EPL; ++j) {
                 const int i = lane + 64 * j;
                 if (i < n) row[i] = v[j];
             }
-            __syncthreads();
+        }
+        __syncthreads();
+        if (qk) {
 #pragma unroll
             for (int j = 0; j < MAX_EPL; ++j) {
                 const int i = lane + 64 * j;
@@ -94,7 +99,8 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
                 }
             }
         }
-    } else if (vf_role) {
+    }
+    if (!qk && vf_role) {
         float* vf = v_first + (size_t)t * nkv * dv + (size_t)kvh * dv;
         const float lam = vf_role == 2 ? lambda[0] : 0.f;
 #pragma unroll
@@ -115,6 +121,51 @@ __global__ __launch_bounds__(64) void pwa_prepare_kernel(
     }
 }
 
+// The values of a step of many tokens: a workgroup takes 64 packed tokens x 64 channels of one kv head through
+// an LDS tile, so that the float sums are read in rows (bias, mixing and `v_first` as in `prepare`) and the
+// transposed values are stored 64 neighbouring tokens of a channel at a time.  grid (ceil(T / 64), nkv,
+// ceil(dv / 64)), block 256.
+template <typename T>
+__global__ __launch_bounds__(256) void pwa_values_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ pos,
+    const int* __restrict__ seq_of_token, const int* __restrict__ slots, const int* __restrict__ block_table,
+    int table_stride, T* __restrict__ storage, float* __restrict__ v_first, const float* __restrict__ lambda,
+    int vf_role, int n_tokens, int nq, int nkv, int dk, int dv, int page) {
+    __shared__ float tile[64][65];
+    const int t0 = blockIdx.x * 64, kvh = blockIdx.y, c0 = blockIdx.z * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int width = nq * dk + nkv * dk + nkv * dv;
+    const int col0 = nq * dk + nkv * dk + kvh * dv;
+    const float lam = vf_role == 2 ? lambda[0] : 0.f;
+    const int ch = c0 + lane;
+    for (int r = 0; r < 16; ++r) {
+        const int tt = wave + 4 * r, t = t0 + tt;
+        float v = 0.f;
+        if (t < n_tokens && ch < dv) {
+            v = qkv[(size_t)t * width + col0 + ch] + (bias ? bias[col0 + ch] : 0.f);
+            if (vf_role) {
+                float* vf = v_first + (size_t)t * nkv * dv + (size_t)kvh * dv + ch;
+                if (vf_role == 1) *vf = v;
+                else v = (1.0f - lam) * v + lam * *vf;
+            }
+        }
+        tile[tt][lane] = v;
+    }
+    __syncthreads();
+    const int t = t0 + lane;
+    if (t >= n_tokens) return;
+    const int slot = slots[seq_of_token[t]];
+    if (slot < 0) return;
+    const int p = pos[t];
+    const size_t page_elems = (size_t)nkv * page * (dk + dv);
+    T* dst = storage + (size_t)block_table[(size_t)slot * table_stride + p / page] * page_elems + (size_t)nkv * page * dk +
+             (size_t)kvh * dv * page + (p % page);
+    for (int r = 0; r < 16; ++r) {
+        const int cc = wave + 4 * r;
+        if (c0 + cc < dv) dst[(size_t)(c0 + cc) * page] = from_f32<T>(tile[lane][cc]);
+    }
+}
+
 extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* qn_w, const float* kn_w, float eps,
                               const float* cs, const float* sn, int rd, const int* pos, const int* seq_of_token,
                               const int* slots, const int* block_table, int table_stride, void* q_out,
@@ -125,7 +176,9 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
         rd < 0 || rd > dk || (rd & 1) || page <= 0 || nq + 2 * nkv > 65535 || (rd > 0 && (!cs || !sn)) ||
         (vf_role && !v_first) || (vf_role == 2 && !lambda) || vf_role < 0 || vf_role > 2)
         return BR_BAD_ARG;
-    dim3 grid(T, nq + 2 * nkv);
+    // steps of many tokens that store their values: the values by the tile kernel
+    const bool tiled = T >= 256 && write_cache;
+    dim3 grid(T, nq + nkv + (tiled ? 0 : nkv));
     const size_t lds = (size_t)(dk > dv ? dk : dv) * sizeof(float);
     if (is_bf16)
         pwa_prepare_kernel<bf16><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
@@ -135,6 +188,15 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
         pwa_prepare_kernel<float><<<grid, 64, lds, s>>>(qkv, bias, qn_w, kn_w, eps, cs, sn, rd, pos, seq_of_token, slots,
                                                         block_table, table_stride, (float*)q_out, (float*)storage,
                                                         v_first, lambda, vf_role, nq, nkv, dk, dv, page, write_cache);
+    int rc = br_check_launch();
+    if (rc != BR_OK || !tiled) return rc;
+    dim3 vgrid((T + 63) / 64, nkv, (dv + 63) / 64);
+    if (is_bf16)
+        pwa_values_kernel<bf16><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (bf16*)storage,
+                                                      v_first, lambda, vf_role, T, nq, nkv, dk, dv, page);
+    else
+        pwa_values_kernel<float><<<vgrid, 256, 0, s>>>(qkv, bias, pos, seq_of_token, slots, block_table, table_stride, (float*)storage,
+                                                       v_first, lambda, vf_role, T, nq, nkv, dk, dv, page);
     return br_check_launch();
 }
 
@@ -380,13 +442,15 @@ __device__ __forceinline__ bf16x8 pwa_load_vt8(const bf16* __restrict__ vrow, in
 // acc[r] the key 16 (r / 8) + 8 g + r % 8.
 __device__ __forceinline__ int pwa_key_of_row(int c) { return 16 * (c >> 4) + 8 * ((c >> 2) & 1) + 4 * ((c >> 3) & 1) + (c & 3); }
 
-// One block of 32 keys (rows kb .. kb + 31 of a unit, kl = kb % 64 within the page `pg`): a key is
-// seen by this lane's query if first_ok <= key <= last_ok.
+// One block of 32 keys (rows kb .. kb + 31 of a unit): `kblock` is the block's first key row (rows `ks` elements
+// apart), `vblock` the first value channel at the block's first row (channels `vs` elements apart), in the cache
+// or in LDS; rows of the block from `limit` on are not written and their values read as zero.  A key is seen by
+// this lane's query if first_ok <= key <= last_ok.
 template <int NBK, int NBV>
-__device__ __forceinline__ void pwa_block(const bf16* __restrict__ pg, size_t k_off, size_t v_off, int kb, int kl,
-                                          int limit, int first_ok, int last_ok, int dk, int dv, int c, int g,
+__device__ __forceinline__ void pwa_block(const bf16* __restrict__ kblock, int ks, const bf16* __restrict__ vblock, int vs,
+                                          int kb, int limit, int first_ok, int last_ok, int dk, int dv, int c, int g,
                                           const bf16x8* qf, f32x16* acc_o, float& m, float& lsum, float scale2) {
-    const bf16* krow = pg + k_off + (size_t)(kl + pwa_key_of_row(c)) * dk;
+    const bf16* krow = kblock + (size_t)pwa_key_of_row(c) * ks;
     f32x16 s_acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
@@ -398,11 +462,18 @@ __device__ __forceinline__ void pwa_block(const bf16* __restrict__ pg, size_t k_
     }
     float sv[16];
     float mx = -INFINITY;
+    // the mask only where some lane's query does not see the whole block (the window's edges, the last pooled rows)
+    const bool whole = __all(first_ok <= kb && kb + 31 <= last_ok);
+    if (whole) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
-        sv[r] = (key >= first_ok && key <= last_ok) ? s_acc[r] * scale2 : -INFINITY;
-        mx = fmaxf(mx, sv[r]);
+        for (int r = 0; r < 16; ++r) { sv[r] = s_acc[r] * scale2; mx = fmaxf(mx, sv[r]); }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = kb + 16 * (r >> 3) + 8 * g + (r & 7);
+            sv[r] = (key >= first_ok && key <= last_ok) ? s_acc[r] * scale2 : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
+        }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
@@ -417,36 +488,50 @@ __device__ __forceinline__ void pwa_block(const bf16* __restrict__ pg, size_t k_
         if (r < 8) p1[r] = (bf16)p; else p2[r - 8] = (bf16)p;
     }
     lsum = lsum * corr + psum;
+    // the sums so far are scaled only when some lane's maximum moved
+    const bool moved = __any(m_new != m);
     m = m_new;
 #pragma unroll
     for (int i = 0; i < NBV; ++i) {
+        if (moved) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+            for (int r = 0; r < 16; ++r) acc_o[i][r] *= corr;
+        }
         const int ch = i * 32 + c;
         bf16x8 v1 = pwa_zero8(), v2 = pwa_zero8();
         if (ch < dv) {
-            const bf16* vrow = pg + v_off + (size_t)ch * PWA_PAGE;
-            v1 = pwa_load_vt8(vrow, kl + 8 * g, limit);
-            v2 = pwa_load_vt8(vrow, kl + 16 + 8 * g, limit);
+            const bf16* vrow = vblock + (size_t)ch * vs;
+            v1 = pwa_load_vt8(vrow, 8 * g, limit);
+            v2 = pwa_load_vt8(vrow, 16 + 8 * g, limit);
         }
         acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, p1, acc_o[i], 0, 0, 0);
         acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v2, p2, acc_o[i], 0, 0, 0);
     }
 }
 
+// Which tile of 128 rows a workgroup takes: the last tiles (most keys) first, so that the long workgroups start
+// first; when all workgroups are resident at once, two to a compute unit (`pair`), the second half of the kv
+// heads goes from short to long instead: the two workgroups that share a compute unit (their numbers lie half the
+// grid apart) are then a long and a short one.
+__device__ __forceinline__ int pwa_tile(int pair) {
+    return (pair && ((blockIdx.y * 2 / gridDim.y) & 1)) ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+}
+
+// Two workgroups a compute unit (two waves a SIMD, so that one fills the other's waits) where the
+// accumulators and operands leave room for it: keys and values up to 128 wide.
 template <int NBK, int NBV>
-__global__ __launch_bounds__(256) void pwa_prefill_kernel(
+__global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_prefill_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, int pair) {
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
     const int G = nq / nkv;
     const int rows_total = n_new * G;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int row0 = blockIdx.x * 128 + wave * 32;
+    const int row0 = pwa_tile(pair) * 128 + wave * 32;
     if (row0 >= rows_total) return;
     const int c = lane & 31, g = lane >> 5;
     const int row = row0 + c;
@@ -492,7 +577,8 @@ __global__ __launch_bounds__(256) void pwa_prefill_kernel(
         for (int kb = 0; kb < seen_max; kb += 32) {
             const int kl = kb % PWA_PAGE;
             const bf16* pg = pooled + (size_t)pt[kb / PWA_PAGE] * page_elems;
-            pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, written - (kb - kl), 0, seen - 1, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+            pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, written - kb, 0, seen - 1, dk, dv, c, g,
+                                qf, acc_o, m, lsum, scale2);
         }
     }
     const int* bt = block_table + (size_t)slot * table_stride;
@@ -502,7 +588,8 @@ __global__ __launch_bounds__(256) void pwa_prefill_kernel(
     for (int kb = (lo / 32) * 32; kb <= pq_max; kb += 32) {
         const int kl = kb % PWA_PAGE;
         const bf16* pg = storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
-        pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, ctx - (kb - kl), first_ok, last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+        pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, ctx - kb, first_ok, last_ok, dk, dv, c, g,
+                            qf, acc_o, m, lsum, scale2);
     }
     lsum += __shfl_xor(lsum, 32, 64);
     if (!row_ok) return;
@@ -581,7 +668,8 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
         const bf16* pg = far ? pooled + (size_t)pt[kb / PWA_PAGE] * page_elems : storage + (size_t)bt[kb / PWA_PAGE] * page_elems;
         const int limit = (far ? ctx / pool : ctx) - (kb - kl);
         const int first_ok = row_ok ? (far ? 0 : lo) : 1, last_ok = row_ok ? (far ? seen - 1 : pq) : 0;
-        pwa_block<NBK, NBV>(pg, k_off, v_off, kb, kl, limit, first_ok, last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+        pwa_block<NBK, NBV>(pg + k_off + (size_t)kl * dk, dk, pg + v_off + kl, PWA_PAGE, kb, limit - kl, first_ok, last_ok, dk, dv, c, g,
+                            qf, acc_o, m, lsum, scale2);
     }
     lsum += __shfl_xor(lsum, 32, 64);
     // merge: [wave][2 G lanes] of m and l, [wave][NBV * 16][2 G lanes] of O
@@ -676,11 +764,177 @@ extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, co
 #undef PWA_K
 }
 
+// The same with a page's keys and values staged in LDS once for the workgroup's 128 rows: the pages its rows
+// can see (pooled pages, then token pages) are walked by all four waves together; while a page is multiplied the
+// next one is on its way from the cache into registers (16 bytes a lane and load, whole lines), and goes into
+// the other LDS stage behind the page's one barrier.  Key rows lie PWA_PAD elements further apart than their
+// width and value channels 64 + PWA_PAD apart, so that the 16-byte operand reads of a wave spread over the banks.
+// A wave skips the blocks of a page that none of its own rows sees.
+#define PWA_PAD 8
+
+template <int NBK, int NBV>
+__global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_prefill_lds_kernel(
+    const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
+    int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, int pair) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char pwa_lds[];
+    const int b = blockIdx.z, kvh = blockIdx.y;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
+    const int G = nq / nkv;
+    const int rows_total = n_new * G;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wg_row0 = pwa_tile(pair) * 128;
+    if (wg_row0 >= rows_total) return;                       // the whole workgroup
+    const int row0 = wg_row0 + wave * 32;
+    const bool wave_on = row0 < rows_total;
+    const int c = lane & 31, g = lane >> 5;
+    const int row = row0 + c;
+    const bool row_ok = wave_on && row < rows_total;
+    const int rr = row_ok ? row : rows_total - 1;
+    const int tok = rr / G, head = kvh * G + rr % G;
+    bf16* orow = out + ((size_t)(t0 + tok) * nq + head) * dv;
+    if (slot < 0) {       // padding: no cache behind it
+        if (row_ok && g == 0) for (int d = 0; d < dv; ++d) orow[d] = (bf16)0.f;
+        return;
+    }
+    const int ctx = ctx_lens[b], start = ctx - n_new;
+    const int pq = start + tok;
+    // positions of this wave's rows and of the workgroup's
+    const int last_row = (row0 + 31 < rows_total ? row0 + 31 : rows_total - 1);
+    const int pq_min = start + (wave_on ? row0 : wg_row0) / G, pq_max = start + (wave_on ? last_row : wg_row0) / G;
+    const int wg_last = (wg_row0 + 127 < rows_total ? wg_row0 + 127 : rows_total - 1);
+    const int wg_min = start + wg_row0 / G, wg_max = start + wg_last / G;
+
+    const bf16* qrow = q + ((size_t)(t0 + tok) * nq + head) * dk;
+    bf16x8 qf[2 * NBK];
+#pragma unroll
+    for (int s = 0; s < 2 * NBK; ++s) {
+        const int d = s * 16 + 8 * g;
+        qf[s] = (d < dk) ? *(const bf16x8*)(qrow + d) : pwa_zero8();
+    }
+    f32x16 acc_o[NBV];
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
+    float m = sink ? 0.f : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
+    const float scale2 = scale * PWA_LOG2E;
+    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
+    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+
+    // what the wave's rows see, and the pages the workgroup walks
+    auto seen_of = [&](int p) { const int far = p - size - pool + 1; return (pool > 0 && far >= 0) ? far / pool + 1 : 0; };
+    const int seen = row_ok ? seen_of(pq) : 0, seen_wave = wave_on ? seen_of(pq_max) : 0;
+    const int far_pages = (seen_of(wg_max) + PWA_PAGE - 1) / PWA_PAGE;
+    int wg_lo = wg_min - size + 1;
+    if (wg_lo < 0) wg_lo = 0;
+    int lo_wave = pq_min - size + 1;
+    if (lo_wave < 0) lo_wave = 0;
+    const int first_page = wg_lo / PWA_PAGE;
+    const int n_pages = far_pages + wg_max / PWA_PAGE - first_page + 1;
+    const int written_far = pool > 0 ? ctx / pool : 0;
+    const int first_ok = row_ok ? pq - size + 1 : 1, last_ok = row_ok ? pq : 0;
+    const int* bt = block_table + (size_t)slot * table_stride;
+    const int* pt = pooled_table ? pooled_table + (size_t)slot * pooled_stride : nullptr;
+
+    const int ks = dk + PWA_PAD, vs = PWA_PAGE + PWA_PAD;
+    const size_t stage_elems = (size_t)PWA_PAGE * ks + (size_t)dv * vs;
+    bf16* stage0 = (bf16*)pwa_lds;
+    // a page's keys are PAGE * dk / 8 pieces of 16 bytes, its values dv * 8: each thread brings up to NBK + NBV of each
+    const int k_pieces = PWA_PAGE * dk / 8, v_pieces = dv * 8;
+    bf16x8 rk[NBK], rv[NBV];
+    auto page_of = [&](int n) -> const bf16* {
+        return n < far_pages ? pooled + (size_t)pt[n] * page_elems : storage + (size_t)bt[first_page + (n - far_pages)] * page_elems;
+    };
+    auto fetch = [&](int n) {
+        const bf16* pg = page_of(n);
+#pragma unroll
+        for (int i = 0; i < NBK; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            rk[i] = piece < k_pieces ? *(const bf16x8*)(pg + k_off + (size_t)piece * 8) : pwa_zero8();
+        }
+#pragma unroll
+        for (int i = 0; i < NBV; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            rv[i] = piece < v_pieces ? *(const bf16x8*)(pg + v_off + (size_t)piece * 8) : pwa_zero8();
+        }
+    };
+    auto put = [&](int buf) {
+        bf16* st = stage0 + (size_t)buf * stage_elems;
+        const int per_row = dk / 8;
+#pragma unroll
+        for (int i = 0; i < NBK; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            if (piece < k_pieces) *(bf16x8*)(st + (size_t)(piece / per_row) * ks + (piece % per_row) * 8) = rk[i];
+        }
+        bf16* sv = st + (size_t)PWA_PAGE * ks;
+#pragma unroll
+        for (int i = 0; i < NBV; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            if (piece < v_pieces) *(bf16x8*)(sv + (size_t)(piece >> 3) * vs + (piece & 7) * 8) = rv[i];
+        }
+    };
+    fetch(0);
+    put(0);
+    __syncthreads();
+    for (int n = 0; n < n_pages; ++n) {
+        const int buf = n & 1;
+        if (n + 1 < n_pages) fetch(n + 1);
+        const bf16* st = stage0 + (size_t)buf * stage_elems;
+        const bf16* sv = st + (size_t)PWA_PAGE * ks;
+        const bool far = n < far_pages;
+        const int page_row0 = (far ? n : first_page + (n - far_pages)) * PWA_PAGE;
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            const int kb = page_row0 + 32 * hb;
+            const bool mine = wave_on && (far ? kb < seen_wave : (kb + 31 >= lo_wave && kb <= pq_max));     // wave-uniform
+            if (mine)
+                pwa_block<NBK, NBV>(st + (size_t)(32 * hb) * ks, ks, sv + 32 * hb, vs, kb, (far ? written_far : ctx) - kb,
+                                    far ? 0 : first_ok, far ? seen - 1 : last_ok, dk, dv, c, g, qf, acc_o, m, lsum, scale2);
+        }
+        if (n + 1 < n_pages) put(buf ^ 1);
+        __syncthreads();
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!row_ok) return;
+    const float inv = lsum > 0.f ? 1.f / lsum : 0.f;
+#pragma unroll
+    for (int i = 0; i < NBV; ++i)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int d = i * 32 + 8 * r4 + 4 * g;
+            if (d < dv) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (bf16)(acc_o[i][4 * r4 + e] * inv);
+                *(bf16x4*)(orow + d) = o;
+            }
+        }
+}
+
 template <int NBK>
 static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
                                 const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
                                 int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
-#define PWA_GO(V) pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink)
+    // steps that fill a workgroup's 128 rows stage the pages in LDS (key widths in steps of 8 and value widths in steps
+    // of 8 that the kernel's pieces cover); shorter ones read their operands straight from the cache
+    const int cus = br_device_cus();
+    const int pair = cus > 0 && (long long)grid.x * grid.y * grid.z <= 2LL * cus;
+    const bool staged = (long long)grid.x * 128 >= 256 && dv % 8 == 0 && dk <= NBK * 32 && dk * 8 <= NBK * 256;
+    const size_t lds = (size_t)2 * ((size_t)PWA_PAGE * (dk + PWA_PAD) + (size_t)dv * (PWA_PAGE + PWA_PAD)) * sizeof(bf16);
+#define PWA_GO(V) do { \
+        if (staged && dv * 8 <= V * 256) { \
+            auto kern = pwa_prefill_lds_kernel<NBK, V>; \
+            static size_t have = 0; \
+            if (lds > have) { \
+                if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
+                have = lds; \
+            } \
+            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, pair); \
+        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, pair); \
+    } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
     else if (nbv <= 3) PWA_GO(3);
