@@ -206,12 +206,12 @@ extern "C" int br_pwa_prepare(const float* qkv, const float* bias, const float* 
 // into row b of the pooled unit.  Block floor(start / pool) + blockIdx.y is this workgroup's;
 // the grid's second size is max_new / pool + 1.
 template <typename T>
-__global__ __launch_bounds__(64) void pwa_pool_kernel(
+__global__ __launch_bounds__(256) void pwa_pool_kernel(
     const T* __restrict__ storage, const int* __restrict__ block_table, int table_stride,
     T* __restrict__ pooled, const int* __restrict__ pooled_table, int pooled_stride,
     const int* __restrict__ cu_seqlens, const int* __restrict__ ctx_lens, const int* __restrict__ slots,
     int nkv, int dk, int dv, int page, int pool) {
-    const int s = blockIdx.x, kvh = blockIdx.z, lane = threadIdx.x;
+    const int s = blockIdx.x, kvh = blockIdx.z;
     const int slot = slots[s];
     if (slot < 0) return;
     const int end = ctx_lens[s];
@@ -224,14 +224,25 @@ __global__ __launch_bounds__(64) void pwa_pool_kernel(
     T* pk = pooled + (size_t)ppg * page_elems + ((size_t)kvh * page + (b % page)) * dk;
     T* pv = pooled + (size_t)ppg * page_elems + (size_t)nkv * page * dk + (size_t)kvh * dv * page + (b % page);
     const float inv = 1.0f / (float)pool;
-    for (int i = lane; i < dk + dv; i += 64) {
+    for (int i = threadIdx.x; i < dk + dv; i += blockDim.x) {      // a channel a lane
         const bool key = i < dk;
         float acc = 0.f;
-        for (int r = 0; r < pool; ++r) {
-            const int j = b * pool + r;
-            const T* pb = storage + (size_t)bt[j / page] * page_elems;
-            acc += key ? to_f32<T>(pb[((size_t)kvh * page + (j % page)) * dk + i])
-                       : to_f32<T>(pb[(size_t)nkv * page * dk + ((size_t)kvh * dv + (i - dk)) * page + (j % page)]);
+        // the rows are added in their order; eight are asked for at a time
+        for (int r0 = 0; r0 < pool; r0 += 8) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int r = r0 + u;
+                x[u] = 0.f;
+                if (r < pool) {
+                    const int j = b * pool + r;
+                    const T* pb = storage + (size_t)bt[j / page] * page_elems;
+                    x[u] = key ? to_f32<T>(pb[((size_t)kvh * page + (j % page)) * dk + i])
+                               : to_f32<T>(pb[(size_t)nkv * page * dk + ((size_t)kvh * dv + (i - dk)) * page + (j % page)]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += x[u];
         }
         if (key) pk[i] = from_f32<T>(acc * inv);
         else pv[(size_t)(i - dk) * page] = from_f32<T>(acc * inv);
@@ -247,11 +258,12 @@ extern "C" int br_pwa_pool(const void* storage, const int* block_table, int tabl
     const int per_seq = max_new / pool + 1;
     if (per_seq > 65535) return BR_TOO_LARGE;
     dim3 grid(B, per_seq, nkv);
+    const int threads = dk + dv > 128 ? 256 : (dk + dv > 64 ? 128 : 64);
     if (is_bf16)
-        pwa_pool_kernel<bf16><<<grid, 64, 0, s>>>((const bf16*)storage, block_table, table_stride, (bf16*)pooled, pooled_table,
+        pwa_pool_kernel<bf16><<<grid, threads, 0, s>>>((const bf16*)storage, block_table, table_stride, (bf16*)pooled, pooled_table,
                                                   pooled_stride, cu_seqlens, ctx_lens, slots, nkv, dk, dv, page, pool);
     else
-        pwa_pool_kernel<float><<<grid, 64, 0, s>>>((const float*)storage, block_table, table_stride, (float*)pooled,
+        pwa_pool_kernel<float><<<grid, threads, 0, s>>>((const float*)storage, block_table, table_stride, (float*)pooled,
                                                    pooled_table, pooled_stride, cu_seqlens, ctx_lens, slots, nkv, dk, dv,
                                                    page, pool);
     return br_check_launch();
