@@ -48,7 +48,14 @@ CONFIGS = {
     # a width that is no multiple of 4, value channels that are no multiple of 4, odd query channels
     "d": model(50, 131, [hgrn2(2, 9, 7, mlp=36), attention(8, 1, 8, 12, 11, 2, rot=(6, 300.0), v_mix=True, mlp=36),
                          attention(2, 1, 12, 12, 4, 6, v_mix=True), hgrn2(1, 33, 16, mlp=20)], emb=2.0, out=0.5),
+    # recurrent layers only (no cache unit at all, no position encoding)
+    "e": model(64, 101, [hgrn2(2, 16, 32, mlp=64), hgrn2(4, 8, 16)]),
+    # attention only, keys wider than 128 and values of three blocks of 32; the second layer's config leaves out
+    # kv_heads (= heads) and scale (= 1 / sqrt(dim))
+    "f": model(128, 90, [attention(2, 1, 160, 96, 20, 4, rot=(64, 1e4), mlp=128), attention(4, 4, 16, 16, 9, 0, mlp=64)]),
 }
+for _k in ("kv_heads", "scale"):
+    del CONFIGS["f"]["layers"][1]["mixer"][_k]
 
 
 @pytest.fixture(scope="module")
