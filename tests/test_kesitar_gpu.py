@@ -457,7 +457,7 @@ def test_slots_and_pages_used_again(folders, engines):
     """Requests come and go through a cache of few pages: what a freed slot or a returned page held never shows."""
     import braidinfer_amd as B
     folder, cfg, w = folders["a"]
-    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=640, max_seq_len=512, n_slots=3)
+    eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=704, max_seq_len=512, n_slots=3)
     free_before = [g.pool.free_count for g in eng.cache.groups]
     for r in range(6):
         toks = tokens_of(cfg, 100 + 37 * r, 50 + r)
