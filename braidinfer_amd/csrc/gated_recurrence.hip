@@ -136,32 +136,24 @@ __global__ __launch_bounds__(256) void glr_scan_kernel(
         const bool more = tc0 + TC < t1;
         if (more) fetch(tc0 + TC);
         const int nt = t1 - tc0 < TC ? t1 - tc0 : TC;
-        // the next token's gates, queries and value are asked from LDS before this token's are used
         const float* fp = fL + (size_t)buf * TC * DP + g * RPL;
         const float* qp = qL + (size_t)buf * TC * DP + g * RPL;
         const float* vp = vL + buf * TC * 16 + wave * 4 + cg;
-        f32x4 fc[RPL / 4], qc[RPL / 4];
-        float vc = vp[0];
-#pragma unroll
-        for (int k4 = 0; k4 < RPL / 4; ++k4) { fc[k4] = *(const f32x4*)(fp + 4 * k4); qc[k4] = *(const f32x4*)(qp + 4 * k4); }
+#pragma unroll 4
         for (int tt = 0; tt < nt; ++tt) {
-            const int nx = tt + 1 < TC ? tt + 1 : tt;
-            f32x4 fn[RPL / 4], qn[RPL / 4];
-            const float vn = vp[nx * 16];
-#pragma unroll
-            for (int k4 = 0; k4 < RPL / 4; ++k4) {
-                fn[k4] = *(const f32x4*)(fp + (size_t)nx * DP + 4 * k4);
-                qn[k4] = *(const f32x4*)(qp + (size_t)nx * DP + 4 * k4);
-            }
+            const float vc = vp[tt * 16];
             float sum = 0.f;
 #pragma unroll
             for (int k4 = 0; k4 < RPL / 4; ++k4) {
+                const f32x4 f = *(const f32x4*)(fp + (size_t)tt * DP + 4 * k4);
+                f32x4 qv = {0.f, 0.f, 0.f, 0.f};
+                if (!LOCAL) qv = *(const f32x4*)(qp + (size_t)tt * DP + 4 * k4);
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
                     // f s + (1 - f) v as v + f (s - v): a subtraction and a multiply-add a row
-                    st[4 * k4 + x] = fmaf(fc[k4][x], st[4 * k4 + x] - vc, vc);
-                    if (LOCAL) dec[LOCAL ? 4 * k4 + x : 0] *= fc[k4][x];
-                    else sum = fmaf(st[4 * k4 + x], qc[k4][x], sum);
+                    st[4 * k4 + x] = fmaf(f[x], st[4 * k4 + x] - vc, vc);
+                    if (LOCAL) dec[LOCAL ? 4 * k4 + x : 0] *= f[x];
+                    else sum = fmaf(st[4 * k4 + x], qv[x], sum);
                 }
             }
             if (!LOCAL) {
@@ -169,9 +161,6 @@ __global__ __launch_bounds__(256) void glr_scan_kernel(
                 if (g == 0 && live) orow[0] = sum;
                 orow += (size_t)H * e;
             }
-            vc = vn;
-#pragma unroll
-            for (int k4 = 0; k4 < RPL / 4; ++k4) { fc[k4] = fn[k4]; qc[k4] = qn[k4]; }
         }
         if (more) stage(buf ^ 1);
         __syncthreads();
