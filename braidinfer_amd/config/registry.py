@@ -119,7 +119,18 @@ def config_from_dict(d: Dict[str, Any]):
 
 
 def config_from_folder(folder: str):
-    return config_from_dict(read_config_json(folder))
+    """The folder's configuration.  A configuration class whose config.json leaves some sizes to the tensors
+    (`missing_tensor_sizes()` names them) gets them from the shapes in the folder's safetensors header
+    (`with_tensor_shapes`); no tensor data is read."""
+    cfg = config_from_dict(read_config_json(folder))
+    missing = getattr(cfg, "missing_tensor_sizes", None)
+    if missing is not None and missing():
+        from ..weights.safetensors_io import SafetensorsFolder
+        st = SafetensorsFolder(folder)
+        cfg = cfg.with_tensor_shapes(lambda name: tuple(st.info(name)[1]) if name in st.where else None)
+        for f in st.files:
+            f.close()
+    return cfg
 
 
 def spec_of(config) -> ModelSpec:

@@ -38,6 +38,8 @@ MODULES: Dict[str, List[str]] = {
     "random_weights": ["random_weights.hip"],
     "pooled_attention": ["pooled_attention.hip"],
     "gated_recurrence": ["gated_recurrence.hip"],
+    "latent_attention": ["latent_attention.hip"],
+    "routed_experts": ["routed_experts.hip"],
 }
 HEADERS = ["common.h", "no_alloc.h"]
 

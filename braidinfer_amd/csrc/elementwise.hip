@@ -486,6 +486,45 @@ extern "C" int br_silu_mul(const void* gu, void* a, int is_bf16, int T, int I, h
     return br_check_launch();
 }
 
+// ----------------------------------------------------------- clamped gated unit -----
+// a[t, i] = g sigmoid(alpha g) (u + 1) with g = min(gu[t, i] + b[i], limit) and
+// u = clamp(gu[t, I + i] + b[I + i], -limit, limit), from the float sums gu [T, 2 I] of the fused gate/up
+// product and their biases b [2 I] (null: none); a has the products' type.
+template <typename T>
+__global__ void clamped_glu_kernel(const float* __restrict__ gu, const float* __restrict__ b, T* __restrict__ a,
+                                   int I, size_t n, float limit, float alpha) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    size_t t = i / I, c = i - t * I;
+    float g = gu[t * 2 * I + c] + (b ? b[c] : 0.f), u = gu[t * 2 * I + I + c] + (b ? b[I + c] : 0.f);
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    a[i] = from_f32<T>(g / (1.f + expf(-alpha * g)) * (u + 1.f));
+}
+
+extern "C" int br_clamped_glu(const float* gu, const float* b, void* a, int a_is_bf16, int T, int I, float limit,
+                              float alpha, hipStream_t s) {
+    if (T <= 0 || I <= 0) return BR_OK;
+    size_t n = (size_t)T * I;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (a_is_bf16) clamped_glu_kernel<bf16><<<blocks, 256, 0, s>>>(gu, b, (bf16*)a, I, n, limit, alpha);
+    else clamped_glu_kernel<float><<<blocks, 256, 0, s>>>(gu, b, (float*)a, I, n, limit, alpha);
+    return br_check_launch();
+}
+
+// x[t, i] += b[i]: the bias of a projection that adds into the residual rows.
+__global__ void add_bias_rows_kernel(float* __restrict__ x, const float* __restrict__ b, int H, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += b[i % H];
+}
+
+extern "C" int br_add_bias_rows(float* x, const float* b, int T, int H, hipStream_t s) {
+    if (T <= 0 || H <= 0) return BR_OK;
+    size_t n = (size_t)T * H;
+    add_bias_rows_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, b, H, n);
+    return br_check_launch();
+}
+
 // ---------------------------------------------------------------- residual add -----
 // x[i] += float(y[i])                 reference: op_residual_add, megakernel_ops.hip:1185-1212
 template <typename T>

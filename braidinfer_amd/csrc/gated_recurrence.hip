@@ -318,3 +318,279 @@ extern "C" int br_glr_head_norm(const float* o, const float* w, void* y, int y_i
 #undef GLR_HN
     return br_check_launch();
 }
+
+// =====================================================================================
+// A recurrence with a decay per key channel and a bonus for the current token: for a head with d key
+// channels and e value channels,
+//     o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,      S_t = diag(w_t) S_(t-1) + k_t v_t^T      (S is d x e, from zero)
+// with the decay w_t = exp(-exp(z_t + w0)) in (0, 1) per channel made on the way into LDS from the float sums
+// z_t of its projection, the receptance r, the key k and the bonus u (one number per head and key channel).
+// Columns of S never meet, so the work is cut like `glr_scan_kernel`'s, the state lies in a slot as that
+// kernel keeps it, and the walk is the same: TC tokens at a time through two LDS stages, the next chunk's rows
+// in flight, a lane holding RPL rows of one column.  A token costs a lane 3 RPL / 4 reads of 16 bytes from LDS,
+// one value, 4 RPL multiply-adds and the four moves that add the row groups' shares of o_t[c].
+//
+// rows [T, width] hold r | k | v | z at the column offsets 0, H d, 2 H d, 2 H d + H e (floats).
+template <int RPL, int TC, bool V4>
+__global__ __launch_bounds__(256) void wkv_scan_kernel(
+    const float* __restrict__ rows, const float* __restrict__ w0, const float* __restrict__ bonus,
+    float* __restrict__ o, float* __restrict__ state, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ slots, int H, int d, int e, int width, size_t slot_stride) {
+    constexpr int DP = RPL * 16;
+    constexpr int NL = TC * DP / 1024;
+    extern __shared__ float lds[];
+    float* wL = lds;                               // [2][TC][DP] decays
+    float* kL = wL + 2 * TC * DP;                  // [2][TC][DP] keys
+    float* rL = kL + 2 * TC * DP;                  // [2][TC][DP] receptances
+    float* vL = rL + 2 * TC * DP;                  // [2][TC][16]
+    const int s = blockIdx.x, h = blockIdx.y, cb16 = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cg = lane >> 4, g = lane & 15;
+    const int cb4 = cb16 * 4 + wave, c = cb4 * 4 + cg;
+    const int slot = slots[s];
+    if (slot < 0) return;
+    const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
+    const bool live = c < e;
+    const int ncb4 = (e + 3) >> 2;
+    float* S = state + (size_t)slot * slot_stride + (((size_t)h * ncb4 + cb4) * RPL) * 64 + lane;
+    float st[RPL], ub[RPL];
+#pragma unroll
+    for (int k = 0; k < RPL; ++k) {
+        st[k] = cb4 < ncb4 ? S[(size_t)k * 64] : 0.f;
+        const int r = g * RPL + k;
+        ub[k] = r < d ? bonus[h * d + r] : 0.f;
+    }
+    const int hd = H * d, he = H * e;
+    int l_tt[NL], l_r4[NL];
+    float b4[NL][4];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int idx = tid + 256 * i;
+        l_tt[i] = idx / (DP / 4);
+        l_r4[i] = (idx % (DP / 4)) * 4;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const int r = l_r4[i] + x;
+            b4[i][x] = r < d ? w0[h * d + r] : 0.f;
+        }
+    }
+    const int v_tt = tid >> 4, v_c = cb16 * 16 + (tid & 15);
+    float rr[NL][4], rk[NL][4], rz[NL][4], rv = 0.f;
+
+    auto fetch = [&](int tc0) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int t = tc0 + l_tt[i];
+            const float* rp = rows + (size_t)t * width + h * d + l_r4[i];
+            const float* zp = rows + (size_t)t * width + 2 * hd + he + h * d + l_r4[i];
+            if (V4) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f}, b = a, z = a;
+                if (t < t1 && l_r4[i] < d) { a = *(const f32x4*)rp; b = *(const f32x4*)(rp + hd); z = *(const f32x4*)zp; }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) { rr[i][x] = a[x]; rk[i][x] = b[x]; rz[i][x] = z[x]; }
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const bool ok = t < t1 && l_r4[i] + x < d;
+                    rr[i][x] = ok ? rp[x] : 0.f;
+                    rk[i][x] = ok ? rp[hd + x] : 0.f;
+                    rz[i][x] = ok ? zp[x] : 0.f;
+                }
+            }
+        }
+        const int t = tc0 + v_tt;
+        rv = (v_tt < TC && t < t1 && v_c < e) ? rows[(size_t)t * width + 2 * hd + h * e + v_c] : 0.f;
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            f32x4 wo, ko, ro;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const bool real = l_r4[i] + x < d;
+                wo[x] = real ? expf(-expf(rz[i][x] + b4[i][x])) : 1.f;
+                ko[x] = real ? rk[i][x] : 0.f;
+                ro[x] = real ? rr[i][x] : 0.f;
+            }
+            const size_t at = ((size_t)buf * TC + l_tt[i]) * DP + l_r4[i];
+            *(f32x4*)(wL + at) = wo;
+            *(f32x4*)(kL + at) = ko;
+            *(f32x4*)(rL + at) = ro;
+        }
+        if (v_tt < TC) vL[(buf * TC + v_tt) * 16 + (tid & 15)] = rv;
+    };
+
+    fetch(t0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    float* orow = o + (size_t)t0 * he + h * e + c;
+    for (int tc0 = t0; tc0 < t1; tc0 += TC) {
+        const bool more = tc0 + TC < t1;
+        if (more) fetch(tc0 + TC);
+        const int nt = t1 - tc0 < TC ? t1 - tc0 : TC;
+        const float* wp = wL + (size_t)buf * TC * DP + g * RPL;
+        const float* kp = kL + (size_t)buf * TC * DP + g * RPL;
+        const float* rp = rL + (size_t)buf * TC * DP + g * RPL;
+        const float* vp = vL + buf * TC * 16 + wave * 4 + cg;
+#pragma unroll 2
+        for (int tt = 0; tt < nt; ++tt) {
+            const float vc = vp[tt * 16];
+            float sum = 0.f;
+#pragma unroll
+            for (int k4 = 0; k4 < RPL / 4; ++k4) {
+                const f32x4 wv = *(const f32x4*)(wp + (size_t)tt * DP + 4 * k4);
+                const f32x4 kv4 = *(const f32x4*)(kp + (size_t)tt * DP + 4 * k4);
+                const f32x4 rv4 = *(const f32x4*)(rp + (size_t)tt * DP + 4 * k4);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const float kv = kv4[x] * vc;
+                    sum = fmaf(rv4[x], fmaf(ub[4 * k4 + x], kv, st[4 * k4 + x]), sum);
+                    st[4 * k4 + x] = fmaf(wv[x], st[4 * k4 + x], kv);
+                }
+            }
+            sum = glr_row16_sum(sum);
+            if (g == 0 && live) orow[0] = sum;
+            orow += he;
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    if (cb4 < ncb4) {
+#pragma unroll
+        for (int k = 0; k < RPL; ++k) S[(size_t)k * 64] = st[k];
+    }
+}
+
+// rows [T, width] float: r | k | v | z at 0, H d, 2 H d, 2 H d + H e; w0 and bonus float [H d]; o float [T, H e];
+// `slot_stride`: floats from one slot's state to the next (at least H * ceil(e / 4) * rows per lane * 64).
+extern "C" int br_wkv_scan(const float* rows, const float* w0, const float* bonus, float* o, float* state,
+                           const int* cu_seqlens, const int* slots, int B, int H, int d, int e, int width,
+                           size_t slot_stride, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    const int ncb4 = (e + 3) / 4, rpl = glr_rpl(d);
+    if (H <= 0 || H > 65535 || d <= 0 || e <= 0 || d > 512 || (e + 15) / 16 > 65535 || width < 3 * H * d + H * e ||
+        slot_stride < (size_t)H * ncb4 * rpl * 64 || !w0 || !bonus)
+        return BR_BAD_ARG;
+    dim3 grid(B, H, (e + 15) / 16);
+    const bool v4 = d % 4 == 0 && e % 4 == 0 && width % 4 == 0 && ((uintptr_t)rows % 16) == 0;
+#define WKV_SCAN(R, TC) do { \
+        const size_t lds = (size_t)(6 * TC * R * 16 + 2 * TC * 16) * sizeof(float); \
+        if (v4) wkv_scan_kernel<R, TC, true><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride); \
+        else wkv_scan_kernel<R, TC, false><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride); \
+    } while (0)
+    if (rpl == 4) WKV_SCAN(4, 16);
+    else if (rpl == 8) WKV_SCAN(8, 16);
+    else if (rpl == 16) WKV_SCAN(16, 8);
+    else WKV_SCAN(32, 4);
+#undef WKV_SCAN
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------- shifted mixes --------
+// out[s][t][:] = h[t] + (h'[t] - h[t]) * mu[s] for `n_mix` mixing vectors mu [n_mix, W], with h' the row of the
+// token before in the same sequence; before a step's first token it is the row the sequence's slot keeps
+// (`kept`, float [W] at the start of what `kept + slot * slot_stride` points to; zeros in a new slot).  The
+// differences are float; out has the rows' type.  A sequence that brings one token also leaves its row in the
+// slot here; longer ones by `shift_keep_kernel` behind this one (their first token reads what the last replaces).
+// grid (T, ceil(W / 256)).
+template <typename T>
+__global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ h, const float* __restrict__ mu,
+                                                        T* __restrict__ out, float* __restrict__ kept, size_t slot_stride,
+                                                        const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                                                        const int* __restrict__ slots, int n_tok, int W, int n_mix) {
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    if (i >= W) return;
+    const int b = seq_of_token[t], slot = slots[b];
+    const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+    const float cur = to_f32<T>(h[(size_t)t * W + i]);
+    float prev = 0.f;
+    if (t > t0) prev = to_f32<T>(h[(size_t)(t - 1) * W + i]);
+    else if (slot >= 0) prev = kept[(size_t)slot * slot_stride + i];
+    const float diff = prev - cur;
+    for (int s = 0; s < n_mix; ++s)
+        out[((size_t)s * n_tok + t) * W + i] = from_f32<T>(fmaf(diff, mu[(size_t)s * W + i], cur));
+    if (slot >= 0 && t1 - t0 == 1) kept[(size_t)slot * slot_stride + i] = cur;
+}
+
+// The last row of every sequence that brought more than one token into its slot.  grid (B, ceil(W / 256)).
+template <typename T>
+__global__ __launch_bounds__(256) void shift_keep_kernel(const T* __restrict__ h, float* __restrict__ kept, size_t slot_stride,
+                                                         const int* __restrict__ cu_seqlens, const int* __restrict__ slots, int W) {
+    const int b = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    const int slot = slots[b];
+    const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
+    if (i >= W || slot < 0 || t1 - t0 <= 1) return;
+    kept[(size_t)slot * slot_stride + i] = to_f32<T>(h[(size_t)(t1 - 1) * W + i]);
+}
+
+extern "C" int br_shift_mix(const void* h, int is_bf16, const float* mu, void* out, float* kept, size_t slot_stride,
+                            const int* seq_of_token, const int* cu_seqlens, const int* slots, int T, int B, int W, int n_mix,
+                            int single_tokens, hipStream_t s) {
+    if (T <= 0 || B <= 0) return BR_OK;
+    if (W <= 0 || n_mix <= 0 || !kept || slot_stride < (size_t)W || (W + 255) / 256 > 65535 || B > 65535) return BR_BAD_ARG;
+    dim3 grid(T, (W + 255) / 256), keep_grid(B, (W + 255) / 256);
+    if (is_bf16) shift_mix_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)h, mu, (bf16*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+    else shift_mix_kernel<float><<<grid, 256, 0, s>>>((const float*)h, mu, (float*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+    int rc = br_check_launch();
+    if (rc != BR_OK || single_tokens) return rc;
+    if (is_bf16) shift_keep_kernel<bf16><<<keep_grid, 256, 0, s>>>((const bf16*)h, kept, slot_stride, cu_seqlens, slots, W);
+    else shift_keep_kernel<float><<<keep_grid, 256, 0, s>>>((const float*)h, kept, slot_stride, cu_seqlens, slots, W);
+    return br_check_launch();
+}
+
+// ------------------------------------------------ head norm, weight and gate --------
+// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w[h, :] * silu(gate[t, h, :]): every head's output
+// divided by its root mean square, a weight per head and channel, and a gate from the float sums of its
+// projection (rows `gate_stride` floats apart).  16 lanes a (token, head) row as in `glr_head_norm_kernel`.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                             const float* __restrict__ gate, size_t gate_stride,
+                                                             T* __restrict__ y, size_t n_rows, int H, int e, float eps) {
+    const size_t r = (size_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int l = threadIdx.x & 15;
+    const bool on = r < n_rows;
+    const float* orow = o + (on ? r : 0) * e;
+    float ss = 0.f;
+    for (int i = l; i < e; i += 16) { const float v = on ? orow[i] : 0.f; ss += v * v; }
+    const float inv = 1.0f / sqrtf(glr_row16_sum(ss) / (float)e + eps);
+    if (!on) return;
+    const size_t t = r / H;
+    const int hh = (int)(r - t * H);
+    const float* grow = gate ? gate + t * gate_stride + (size_t)hh * e : nullptr;
+    const float* wrow = w ? w + (size_t)hh * e : nullptr;
+    T* yrow = y + r * e;
+    for (int i = l; i < e; i += 16) {
+        float v = orow[i] * inv;
+        if (wrow) v *= wrow[i];
+        if (grow) { const float z = grow[i]; v *= z / (1.0f + expf(-z)); }
+        yrow[i] = from_f32<T>(v);
+    }
+}
+
+extern "C" int br_head_norm_gate(const float* o, const float* w, const float* gate, size_t gate_stride, void* y, int y_is_bf16,
+                                 int T, int H, int e, float eps, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (H <= 0 || e <= 0 || (gate && gate_stride < (size_t)H * e)) return BR_BAD_ARG;
+    const size_t n_rows = (size_t)T * H;
+    const unsigned blocks = (unsigned)((n_rows + 15) / 16);
+    if (y_is_bf16) head_norm_gate_kernel<bf16><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (bf16*)y, n_rows, H, e, eps);
+    else head_norm_gate_kernel<float><<<blocks, 256, 0, s>>>(o, w, gate, gate_stride, (float*)y, n_rows, H, e, eps);
+    return br_check_launch();
+}
+
+// y = tanh(x) elementwise, float sums in, the products' type out (the middle of a low-rank projection).
+template <typename T>
+__global__ __launch_bounds__(256) void tanh_kernel(const float* __restrict__ x, T* __restrict__ y, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = from_f32<T>(tanhf(x[i]));
+}
+
+extern "C" int br_tanh(const float* x, void* y, int y_is_bf16, size_t n, hipStream_t s) {
+    if (n == 0) return BR_OK;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (y_is_bf16) tanh_kernel<bf16><<<blocks, 256, 0, s>>>(x, (bf16*)y, n);
+    else tanh_kernel<float><<<blocks, 256, 0, s>>>(x, (float*)y, n);
+    return br_check_launch();
+}

@@ -290,7 +290,7 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
     const int* __restrict__ seq_of_token, const int* __restrict__ slots,
     const int* __restrict__ block_table, int table_stride, const T* __restrict__ storage,
     const int* __restrict__ pooled_table, int pooled_stride, const T* __restrict__ pooled,
-    int nq, int nkv, int dk, int dv, int page, int size, int pool, float scale, int sink) {
+    int nq, int nkv, int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
     extern __shared__ float lds[];
     float* qs = lds;                         // [dk]
     float* ps = qs + dk;                     // [4][64]
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
     const size_t k_off = (size_t)kvh * page * dk, v_off = (size_t)nkv * page * dk + (size_t)kvh * dv * page;
     float* pw = ps + wave * 64;
 
-    float m = (sink && wave == 0) ? 0.f : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
+    float m = (sink && wave == 0) ? (sinks ? sinks[h] : 0.f) : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
     float acc[MAX_EPL];
 #pragma unroll
     for (int i = 0; i < MAX_EPL; ++i) acc[i] = 0.f;
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(256) void pwa_attend_kernel(
 extern "C" int br_pwa_attend(const void* q, void* out, int is_bf16, const int* pos, const int* seq_of_token,
                              const int* slots, const int* block_table, int table_stride, const void* storage,
                              const int* pooled_table, int pooled_stride, const void* pooled, int T, int nq, int nkv,
-                             int dk, int dv, int page, int size, int pool, float scale, int sink, hipStream_t s) {
+                             int dk, int dv, int page, int size, int pool, float scale, int sink, const float* __restrict__ sinks, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || dk <= 0 || dv <= 0 || dk > 64 * MAX_EPL || dv > 64 * MAX_EPL || page != 64 ||
         size <= 0 || pool < 0 || nq > 65535 || (pool > 0 && (!pooled_table || !pooled)))
@@ -415,7 +415,7 @@ extern "C" int br_pwa_attend(const void* q, void* out, int is_bf16, const int* p
     // 16-byte loads where every row starts at a multiple of 16 bytes
     const bool vec = is_bf16 ? dk % 8 == 0 : dk % 4 == 0;
 #define PWA_ATT(TT, V) pwa_attend_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)q, (TT*)out, pos, seq_of_token, slots, block_table, \
-        table_stride, (const TT*)storage, pooled_table, pooled_stride, (const TT*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink)
+        table_stride, (const TT*)storage, pooled_table, pooled_stride, (const TT*)pooled, nq, nkv, dk, dv, page, size, pool, scale, sink, sinks)
     if (is_bf16) { if (vec) PWA_ATT(bf16, true); else PWA_ATT(bf16, false); }
     else { if (vec) PWA_ATT(float, true); else PWA_ATT(float, false); }
 #undef PWA_ATT
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, int pair) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair) {
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
     const int t0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - t0;
@@ -574,7 +574,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     // the two lane halves of a query add their sums at the end: the sink's one goes to the first
-    float m = sink ? 0.f : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
+    float m = sink ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
     const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
     const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
@@ -634,7 +634,7 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
     const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
     extern __shared__ float lds[];
     const int b = blockIdx.y, kvh = blockIdx.x;
     const int slot = slots[b];
@@ -660,7 +660,7 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
     for (int i = 0; i < NBV; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
-    float m = (sink && wave == 0) ? 0.f : -INFINITY, lsum = (sink && wave == 0 && g == 0) ? 1.f : 0.f;
+    float m = (sink && wave == 0) ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && wave == 0 && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
     const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
     const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
@@ -733,8 +733,8 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
 template <int NBK>
 static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStream_t s, const bf16* q, bf16* out, const int* slots,
                                const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
-                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, size_t head_lds) {
-#define PWA_GO(V) pwa_decode_kernel<NBK, V><<<grid, 64 * PWA_DW, head_lds + lds_of_nbv16 * V, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink)
+                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds) {
+#define PWA_GO(V) pwa_decode_kernel<NBK, V><<<grid, 64 * PWA_DW, head_lds + lds_of_nbv16 * V, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
     else if (nbv <= 3) PWA_GO(3);
@@ -757,7 +757,7 @@ extern "C" int br_pwa_decode_takes(int nq, int nkv, int dk, int dv) {
 extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, const int* ctx_lens, const int* block_table,
                                   int table_stride, const void* storage, const int* pooled_table, int pooled_stride,
                                   const void* pooled, int B, int nq, int nkv, int dk, int dv, int size, int pool, float scale,
-                                  int sink, hipStream_t s) {
+                                  int sink, const float* __restrict__ sinks, hipStream_t s) {
     if (B <= 0) return BR_OK;
     if (!br_pwa_decode_takes(nq, nkv, dk, dv) || nkv > 65535 || B > 65535 || size <= 0 || pool < 0 ||
         (pool > 0 && (!pooled_table || !pooled)))
@@ -767,7 +767,7 @@ extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, co
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
     const size_t head_lds = (size_t)2 * PWA_DW * 2 * G * sizeof(float), per_v = (size_t)PWA_DW * 16 * 2 * G * sizeof(float);
 #define PWA_K(KK) pwa_decode_launch_v<KK>(nbv, grid, per_v, s, (const bf16*)q, (bf16*)out, slots, ctx_lens, block_table, table_stride, \
-                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, head_lds)
+                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, head_lds)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);
@@ -789,7 +789,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ cu_seqlens,
     const int* __restrict__ slots, const int* __restrict__ ctx_lens, const int* __restrict__ block_table,
     int table_stride, const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, int pair) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int pair) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pwa_lds[];
     const int b = blockIdx.z, kvh = blockIdx.y;
     const int slot = slots[b];
@@ -831,7 +831,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
     for (int i = 0; i < NBV; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
-    float m = sink ? 0.f : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
+    float m = sink ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
     const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
     const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
@@ -929,7 +929,7 @@ __global__ __launch_bounds__(256, ((NBK <= 4 && NBV <= 4) ? 2 : 1)) void pwa_pre
 template <int NBK>
 static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q, bf16* out, const int* cu, const int* slots,
                                 const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
-                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink) {
+                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
     // steps that fill a workgroup's 128 rows stage the pages in LDS (key widths in steps of 8 and value widths in steps
     // of 8 that the kernel's pieces cover); shorter ones read their operands straight from the cache
     const int cus = br_device_cus();
@@ -944,8 +944,8 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
                 if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
                 have = lds; \
             } \
-            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, pair); \
-        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, pair); \
+            kern<<<grid, 256, lds, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair); \
+        } else pwa_prefill_kernel<NBK, V><<<grid, 256, 0, s>>>(q, out, cu, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, pair); \
     } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
@@ -960,7 +960,7 @@ static int pwa_prefill_launch_v(int nbv, dim3 grid, hipStream_t s, const bf16* q
 extern "C" int br_pwa_prefill_bf16(const void* q, void* out, const int* cu_seqlens, const int* slots, const int* ctx_lens,
                                    const int* block_table, int table_stride, const void* storage, const int* pooled_table,
                                    int pooled_stride, const void* pooled, int B, int max_new, int nq, int nkv, int dk, int dv,
-                                   int size, int pool, float scale, int sink, hipStream_t s) {
+                                   int size, int pool, float scale, int sink, const float* __restrict__ sinks, hipStream_t s) {
     if (B <= 0 || max_new <= 0) return BR_OK;
     if (nq <= 0 || nkv <= 0 || nq % nkv || nkv > 65535 || B > 65535 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 ||
         dv % 4 || size <= 0 || pool < 0 || (pool > 0 && (!pooled_table || !pooled)))
@@ -969,7 +969,7 @@ extern "C" int br_pwa_prefill_bf16(const void* q, void* out, const int* cu_seqle
     dim3 grid((unsigned)(((size_t)max_new * G + 127) / 128), nkv, B);
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
 #define PWA_K(KK) pwa_prefill_launch_v<KK>(nbv, grid, s, (const bf16*)q, (bf16*)out, cu_seqlens, slots, ctx_lens, block_table, table_stride, \
-                                           (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink)
+                                           (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);

@@ -1,0 +1,154 @@
+// A feed-forward of routed experts: every token goes through the `top` experts with the largest router
+// scores and takes their outputs weighted by the softmax over those scores only.  An expert is
+// W_d (silu(W_g h) * (W_u h)) without biases; the experts' matrices lie stacked, [E][F][W] for gate and up and
+// [E][W][F] for down.
+//
+//   route:  scores (the router product's float sums) + bias -> the chosen experts and their shares, float;
+//           ties go to the lower expert number.
+//   up:     y[t, s, :] = silu(W_g[e] h_t) * (W_u[e] h_t) for slot s of token t with e its expert.
+//   down:   x[t, :] += sum_s share[t, s] * W_d[e_s] y[t, s, :], slots added in slot order in float.
+// `up` and `down` read an expert's rows once per (token, slot): the form for steps of few tokens, where the
+// experts' weights are what a step reads.
+#include "common.h"
+
+#define RX_MAX_PER_LANE 8          // experts a lane keeps: up to 512 experts
+
+// grid (T), one wave a token.
+__global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict__ scores, const float* __restrict__ bias,
+                                                        int* __restrict__ chosen, float* __restrict__ share, int E, int top) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float z[RX_MAX_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        z[i] = e < E ? scores[(size_t)t * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    }
+    float first = 0.f, total = 0.f, mine = 0.f;
+    for (int s = 0; s < top; ++s) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i) {
+            const int e = lane + 64 * i;
+            if (e < E && (z[i] > best || (z[i] == best && e < at))) { best = z[i]; at = e; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, WAVE);
+            const int oa = __shfl_xor(at, o, WAVE);
+            if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+        }
+        if (s == 0) first = best;                 // the largest score: the softmax's shift
+        const float w = expf(best - first);
+        total += w;
+        if (lane == s) mine = w;                  // lane s keeps slot s's weight
+        if (lane == 0) chosen[(size_t)t * top + s] = at;
+#pragma unroll
+        for (int i = 0; i < RX_MAX_PER_LANE; ++i)
+            if (lane + 64 * i == at) z[i] = -INFINITY;
+    }
+    if (lane < top) share[(size_t)t * top + lane] = mine / total;
+}
+
+extern "C" int br_route_topk(const float* scores, const float* bias, int* chosen, float* share, int T, int E, int top,
+                             hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (E <= 0 || E > 64 * RX_MAX_PER_LANE || top <= 0 || top > E || top > 64) return BR_BAD_ARG;
+    route_topk_kernel<<<T, 64, 0, s>>>(scores, bias, chosen, share, E, top);
+    return br_check_launch();
+}
+
+template <typename T> struct rx_vec;
+template <> struct rx_vec<float> { static constexpr int N = 4; typedef f32x4 type; };
+template <> struct rx_vec<bf16> { static constexpr int N = 8; typedef bf16x8 type; };
+
+// One weight row times the activations in LDS (float), lanes across k; VEC: 16-byte loads.
+template <typename T, bool VEC>
+__device__ __forceinline__ float rx_dot(const T* __restrict__ wrow, const float* __restrict__ a, int K, int lane) {
+    constexpr int VN = rx_vec<T>::N;
+    typedef typename rx_vec<T>::type vec_t;
+    float acc = 0.f;
+    if (VEC) {
+        for (int k = lane * VN; k < K; k += 64 * VN) {
+            const vec_t w = *(const vec_t*)(wrow + k);
+#pragma unroll
+            for (int i = 0; i < VN; ++i) acc = fmaf(to_f32<T>(w[i]), a[k + i], acc);
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) acc = fmaf(to_f32<T>(wrow[k]), a[k], acc);
+    }
+    return wave_sum(acc);
+}
+
+// grid (T * top, ceil(F / 16)), 4 waves, a wave four columns.  LDS: W floats.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void experts_up_kernel(const T* __restrict__ h, const T* __restrict__ w_gate,
+                                                         const T* __restrict__ w_up, const int* __restrict__ chosen,
+                                                         T* __restrict__ y, int W, int F, int top) {
+    extern __shared__ float hs[];
+    const int slot = blockIdx.x, t = slot / top;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < W; i += 256) hs[i] = to_f32<T>(h[(size_t)t * W + i]);
+    __syncthreads();
+    const int e = chosen[slot];
+    const T* wg = w_gate + (size_t)e * F * W;
+    const T* wu = w_up + (size_t)e * F * W;
+    for (int j = 0; j < 4; ++j) {
+        const int f = blockIdx.y * 16 + wave * 4 + j;
+        if (f >= F) break;
+        const float g = rx_dot<T, VEC>(wg + (size_t)f * W, hs, W, lane);
+        const float u = rx_dot<T, VEC>(wu + (size_t)f * W, hs, W, lane);
+        if (lane == 0) y[(size_t)slot * F + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    }
+}
+
+// grid (T, ceil(W / 16)), 4 waves, a wave four columns.  LDS: top * F floats.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__ y, const T* __restrict__ w_down,
+                                                           const int* __restrict__ chosen, const float* __restrict__ share,
+                                                           float* __restrict__ x, int W, int F, int top) {
+    extern __shared__ float ys[];
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < top * F; i += 256) ys[i] = to_f32<T>(y[(size_t)t * top * F + i]);
+    __syncthreads();
+    for (int j = 0; j < 4; ++j) {
+        const int n = blockIdx.y * 16 + wave * 4 + j;
+        if (n >= W) break;
+        float sum = 0.f;
+        for (int s = 0; s < top; ++s) {
+            const int e = chosen[(size_t)t * top + s];
+            const float d = rx_dot<T, VEC>(w_down + ((size_t)e * W + n) * F, ys + (size_t)s * F, F, lane);
+            sum = fmaf(share[(size_t)t * top + s], d, sum);
+        }
+        if (lane == 0) x[(size_t)t * W + n] += sum;
+    }
+}
+
+extern "C" int br_experts_up(const void* h, const void* w_gate, const void* w_up, const int* chosen, void* y, int is_bf16,
+                             int T, int W, int F, int top, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (W <= 0 || F <= 0 || top <= 0 || (size_t)W * 4 > 65536 || (F + 15) / 16 > 65535) return BR_BAD_ARG;
+    dim3 grid((unsigned)((size_t)T * top), (F + 15) / 16);
+    const size_t lds = (size_t)W * sizeof(float);
+    const bool vec = W % (is_bf16 ? 8 : 4) == 0;
+#define RX_UP(TT, V) experts_up_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)h, (const TT*)w_gate, (const TT*)w_up, chosen, (TT*)y, W, F, top)
+    if (is_bf16) { if (vec) RX_UP(bf16, true); else RX_UP(bf16, false); }
+    else { if (vec) RX_UP(float, true); else RX_UP(float, false); }
+#undef RX_UP
+    return br_check_launch();
+}
+
+extern "C" int br_experts_down(const void* y, const void* w_down, const int* chosen, const float* share, float* x, int is_bf16,
+                               int T, int W, int F, int top, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (W <= 0 || F <= 0 || top <= 0 || (size_t)top * F * 4 > 65536 || (W + 15) / 16 > 65535) return BR_BAD_ARG;
+    dim3 grid(T, (W + 15) / 16);
+    const size_t lds = (size_t)top * F * sizeof(float);
+    const bool vec = F % (is_bf16 ? 8 : 4) == 0;
+#define RX_DOWN(TT, V) experts_down_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)y, (const TT*)w_down, chosen, share, x, W, F, top)
+    if (is_bf16) { if (vec) RX_DOWN(bf16, true); else RX_DOWN(bf16, false); }
+    else { if (vec) RX_DOWN(float, true); else RX_DOWN(float, false); }
+#undef RX_DOWN
+    return br_check_launch();
+}

@@ -577,10 +577,18 @@ def pwa_pool(unit: torch.Tensor, block_table: torch.Tensor, pooled: torch.Tensor
              _stream()), "pwa_pool")
 
 
+def _sinks(name: str, sinks: Optional[torch.Tensor], nq: int) -> c_void_p:
+    """A learnt sink score per query head (float32 [nq]) for a softmax with a sink; None: the sink's score is 0."""
+    if sinks is not None:
+        _dev(name, sinks)
+        _req(sinks.dtype == torch.float32 and sinks.numel() == nq, f"{name}: sink scores must be float32 [query heads]")
+    return _ptr(sinks)
+
+
 def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, slots: torch.Tensor,
                block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
                pooled: Optional[torch.Tensor], nq: int, nkv: int, dk: int, dv: int, page: int, size: int, pool: int,
-               scale: float, sink: bool) -> None:
+               scale: float, sink: bool, sinks: Optional[torch.Tensor] = None) -> None:
     """One wave per (query, head), float arithmetic: the window's tokens and the pooled blocks before it."""
     _dev("pwa_attend", q, out, positions, seq_of_token, slots, block_table, unit, pooled_table, pooled)
     T = q.shape[0]
@@ -591,11 +599,11 @@ def pwa_attend(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, seq_
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_attend: pooled unit missing")
         _pwa_unit("pwa_attend", pooled, nkv, dk, dv, page)
     f = _fn("pooled_attention", "br_pwa_attend",
-            [_P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P])
+            [_P, _P, c_int, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, _P])
     _check(f(_ptr(q), _ptr(out), _is_bf16(q, "pwa_attend"), _ptr(positions), _ptr(seq_of_token), _ptr(slots),
              _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
              pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), T, nq, nkv, dk, dv, page, int(size),
-             int(pool), float(scale), int(sink), _stream()), "pwa_attend")
+             int(pool), float(scale), int(sink), _sinks("pwa_attend", sinks, nq), _stream()), "pwa_attend")
 
 
 def pwa_prefill_takes(dtype: torch.dtype, dk: int, dv: int, page: int) -> bool:
@@ -606,7 +614,7 @@ def pwa_prefill_takes(dtype: torch.dtype, dk: int, dv: int, page: int) -> bool:
 def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor,
                      block_table: torch.Tensor, unit: torch.Tensor, pooled_table: Optional[torch.Tensor],
                      pooled: Optional[torch.Tensor], B: int, max_new: int, nq: int, nkv: int, dk: int, dv: int, page: int,
-                     size: int, pool: int, scale: float, sink: bool) -> None:
+                     size: int, pool: int, scale: float, sink: bool, sinks: Optional[torch.Tensor] = None) -> None:
     """Steps of several tokens per sequence on the matrix cores: the same sums as `pwa_attend`, bfloat16 operands,
     float scores and softmax, the weights rounded to bfloat16 for the second product."""
     _dev("pwa_prefill_bf16", q, out, cu_seqlens, slots, ctx_lens, block_table, unit, pooled_table, pooled)
@@ -621,10 +629,10 @@ def pwa_prefill_bf16(q: torch.Tensor, out: torch.Tensor, cu_seqlens: torch.Tenso
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_prefill_bf16: pooled unit missing")
         _pwa_unit("pwa_prefill_bf16", pooled, nkv, dk, dv, page)
     f = _fn("pooled_attention", "br_pwa_prefill_bf16",
-            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P])
+            [_P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 8 + [c_float, c_int, _P, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(cu_seqlens), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit),
              _ptr(pooled_table), pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, max_new, nq, nkv, dk, dv,
-             int(size), int(pool), float(scale), int(sink), _stream()), "pwa_prefill_bf16")
+             int(size), int(pool), float(scale), int(sink), _sinks("pwa_prefill_bf16", sinks, nq), _stream()), "pwa_prefill_bf16")
 
 
 def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, page: int) -> bool:
@@ -638,7 +646,8 @@ def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, pa
 
 def pwa_decode_bf16(q: torch.Tensor, out: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor, block_table: torch.Tensor,
                     unit: torch.Tensor, pooled_table: Optional[torch.Tensor], pooled: Optional[torch.Tensor], B: int, nq: int,
-                    nkv: int, dk: int, dv: int, page: int, size: int, pool: int, scale: float, sink: bool) -> None:
+                    nkv: int, dk: int, dv: int, page: int, size: int, pool: int, scale: float, sink: bool,
+                    sinks: Optional[torch.Tensor] = None) -> None:
     """Steps of one token per sequence on the matrix cores (row b of q is sequence b's token): a workgroup per
     (kv head, sequence) serves all query heads of the kv head."""
     _dev("pwa_decode_bf16", q, out, slots, ctx_lens, block_table, unit, pooled_table, pooled)
@@ -650,10 +659,10 @@ def pwa_decode_bf16(q: torch.Tensor, out: torch.Tensor, slots: torch.Tensor, ctx
     if pool:
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_decode_bf16: pooled unit missing")
         _pwa_unit("pwa_decode_bf16", pooled, nkv, dk, dv, page)
-    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P])
+    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
              pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, nq, nkv, dk, dv, int(size), int(pool),
-             float(scale), int(sink), _stream()), "pwa_decode_bf16")
+             float(scale), int(sink), _sinks("pwa_decode_bf16", sinks, nq), _stream()), "pwa_decode_bf16")
 
 
 # ------------------------------------------------------ gated linear recurrence -----
@@ -729,6 +738,158 @@ def head_rmsnorm(o: torch.Tensor, w: Optional[torch.Tensor], out: torch.Tensor, 
     _req(w is None or (w.dtype == torch.float32 and w.numel() == e), "head_rmsnorm: weight float32 [e]")
     f = _fn("gated_recurrence", "br_glr_head_norm", [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P])
     _check(f(_ptr(o), _ptr(w), _ptr(out), _is_bf16(out, "head_rmsnorm"), T, H, e, float(eps), _stream()), "head_rmsnorm")
+
+
+# ------------------------------------------------- decayed recurrence with a bonus -----
+def wkv_scan(rows: torch.Tensor, w0: torch.Tensor, bonus: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+             cu_seqlens: torch.Tensor, slots: torch.Tensor, B: int, H: int, d: int, e: int) -> None:
+    """rows [T, >= 3*H*d + H*e] float, the projections' sums r | k | v | z (the decay is exp(-exp(z + w0)), made on the
+    way); bonus float [H*d].  state [slots, n] float with a slot's first prod(glr_state_shape(H, d, e)) floats its S as
+    `glr_scan` keeps it: walks every sequence's new tokens in order, o_t = (S + diag(bonus) k v^T)^T r before
+    S <- diag(decay) S + k v^T, writes o [T, H*e] float and leaves the state."""
+    _dev("wkv_scan", rows, w0, bonus, out, cu_seqlens, slots)
+    T = rows.shape[0]
+    need = 1
+    for n in glr_state_shape(H, d, e):
+        need *= n
+    _req(state.is_cuda and state.dim() == 2 and state.shape[1] >= need and state.stride(1) == 1,
+         "wkv_scan: state [slots, at least the head states' floats], every slot's dense")
+    _req(rows.dtype == out.dtype == state.dtype == torch.float32, "wkv_scan: float32 only")
+    _req(rows.dim() == 2 and rows.shape[1] >= 3 * H * d + H * e and out.shape == (T, H * e), "wkv_scan: rows [T, >= 3*H*d + H*e], out [T, H*e]")
+    for v in (w0, bonus):
+        _req(v.dtype == torch.float32 and v.numel() == H * d, "wkv_scan: w0 and bonus float32 [H*d]")
+    _req(cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "wkv_scan: arrays shorter than the batch")
+    _req(d <= 512, f"wkv_scan: {d} key channels a head are beyond the kernel's 512")
+    f = _fn("gated_recurrence", "br_wkv_scan", [_P, _P, _P, _P, _P, _P, _P] + [c_int] * 5 + [c_size_t, _P])
+    _check(f(_ptr(rows), _ptr(w0), _ptr(bonus), _ptr(out), _ptr(state), _ptr(cu_seqlens), _ptr(slots), B, H, d, e,
+             rows.shape[1], state.stride(0), _stream()), "wkv_scan")
+
+
+def shift_mix(h: torch.Tensor, mu: torch.Tensor, out: torch.Tensor, kept: torch.Tensor, seq_of_token: torch.Tensor,
+              cu_seqlens: torch.Tensor, slots: torch.Tensor, B: int, single_tokens: bool) -> None:
+    """out[s, t] = h[t] + (h'[t] - h[t]) * mu[s], h' the row of the token before in its sequence, and before a step's
+    first token the row its slot keeps (`kept` [slots, >= W] float, a slot's first W floats); every sequence's last
+    row is left there.  h and out [n, T, W] have the products' type, mu [n, W] is float."""
+    _dev("shift_mix", h, mu, out, seq_of_token, cu_seqlens, slots)
+    T, W = h.shape
+    n = mu.shape[0]
+    _req(mu.dtype == torch.float32 and mu.shape == (n, W) and out.shape == (n, T, W) and out.dtype == h.dtype, "shift_mix: mu float32 [n, W], out [n, T, W] of h's type")
+    _req(kept.is_cuda and kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] >= W and kept.stride(1) == 1, "shift_mix: kept float32 [slots, >= W]")
+    _req(seq_of_token.numel() >= T and cu_seqlens.numel() >= B + 1 and slots.numel() >= B, "shift_mix: arrays shorter than the step")
+    f = _fn("gated_recurrence", "br_shift_mix", [_P, c_int, _P, _P, _P, c_size_t, _P, _P, _P] + [c_int] * 5 + [_P])
+    _check(f(_ptr(h), _is_bf16(h, "shift_mix"), _ptr(mu), _ptr(out), _ptr(kept), kept.stride(0), _ptr(seq_of_token), _ptr(cu_seqlens),
+             _ptr(slots), T, B, W, n, int(single_tokens), _stream()), "shift_mix")
+
+
+def head_norm_gate(o: torch.Tensor, w: Optional[torch.Tensor], gate: Optional[torch.Tensor], out: torch.Tensor, H: int, e: int,
+                   eps: float) -> None:
+    """out[t, h, :] = o[t, h, :] / rms * w[h, :] * silu(gate[t, h, :]): o float [T, H*e], w float [H*e] or None, gate a float
+    view [T, H*e] whose rows may be strided (the sums of its projection) or None."""
+    _dev("head_norm_gate", o, w, out)
+    T = o.shape[0]
+    _req(o.dtype == torch.float32 and o.shape == (T, H * e) and out.shape == (T, H * e), "head_norm_gate: o float32 [T, H*e]")
+    _req(w is None or (w.dtype == torch.float32 and w.numel() == H * e), "head_norm_gate: weight float32 [H*e]")
+    gs = 0
+    if gate is not None:
+        _req(gate.is_cuda and gate.dtype == torch.float32 and gate.shape == (T, H * e) and gate.stride(1) == 1, "head_norm_gate: gate float32 [T, H*e]")
+        gs = gate.stride(0) if T > 1 else H * e
+    f = _fn("gated_recurrence", "br_head_norm_gate", [_P, _P, _P, c_size_t, _P, c_int, c_int, c_int, c_int, c_float, _P])
+    _check(f(_ptr(o), _ptr(w), _ptr(gate), gs, _ptr(out), _is_bf16(out, "head_norm_gate"), T, H, e, float(eps), _stream()), "head_norm_gate")
+
+
+def tanh(x: torch.Tensor, out: torch.Tensor) -> None:
+    _dev("tanh", x, out)
+    _req(x.dtype == torch.float32 and x.numel() == out.numel(), "tanh: x float32, out of the same size")
+    f = _fn("gated_recurrence", "br_tanh", [_P, _P, c_int, c_size_t, _P])
+    _check(f(_ptr(x), _ptr(out), _is_bf16(out, "tanh"), x.numel(), _stream()), "tanh")
+
+
+# ------------------------------------------------------ attention through a latent -----
+def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], c_weight: Optional[torch.Tensor], eps: float,
+                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot: int, positions: torch.Tensor,
+                   seq_of_token: torch.Tensor, slots: torch.Tensor, block_table: Optional[torch.Tensor],
+                   cache: Optional[torch.Tensor], q_plain: torch.Tensor, q_wide: torch.Tensor, H: int, D: int, DR: int, R: int,
+                   page: int) -> None:
+    """q float [T, H*(D+DR)] and dkv float [T, R+DR] (views whose rows may be strided; dkv None: nothing is kept):
+    the normed latent and the rotated shared key part into the token's cache row, the queries' plain parts into
+    q_plain [T, H*D] and their rotated parts into q_wide [T, H*(R+DR)] behind each head's first R elements."""
+    _dev("latent_prepare", c_weight, cos, sin, positions, seq_of_token, slots, block_table, cache, q_plain, q_wide)
+    T = q.shape[0]
+    _req(q.is_cuda and q.dtype == torch.float32 and q.shape == (T, H * (D + DR)) and q.stride(1) == 1, "latent_prepare: q float32 [T, H*(D+DR)]")
+    _req(q_plain.shape == (T, H * D) and q_wide.shape == (T, H * (R + DR)) and q_plain.dtype == q_wide.dtype, "latent_prepare: q_plain [T, H*D], q_wide [T, H*(R+DR)]")
+    if rot:
+        _req(cos is not None and sin is not None and cos.numel() >= T * (rot // 2) and sin.numel() >= T * (rot // 2), "latent_prepare: rotary tables too short")
+    ds = 0
+    if dkv is not None:
+        _req(dkv.is_cuda and dkv.dtype == torch.float32 and dkv.shape == (T, R + DR) and dkv.stride(1) == 1, "latent_prepare: dkv float32 [T, R+DR]")
+        _req(c_weight is not None and c_weight.dtype == torch.float32 and c_weight.numel() == R, "latent_prepare: the latent's norm weight float32 [R]")
+        _req(cache is not None and cache.dtype == q_plain.dtype and cache.dim() == 2 and cache.shape[1] == page * (2 * R + DR),
+             "latent_prepare: cache [pages, page * (2 R + DR)] of the products' type")
+        _req(block_table is not None and block_table.dim() == 2 and block_table.dtype == torch.int32, "latent_prepare: block table int32 [slots, pages]")
+        ds = dkv.stride(0) if T > 1 else R + DR
+    f = _fn("latent_attention", "br_latent_prepare",
+            [_P, c_size_t, _P, c_size_t, _P, c_float, _P, _P, _P, _P, _P, _P, c_int, _P, _P, _P] + [c_int] * 8 + [_P])
+    _check(f(_ptr(q), q.stride(0) if T > 1 else H * (D + DR), _ptr(dkv), ds, _ptr(c_weight), float(eps), _ptr(cos), _ptr(sin),
+             _ptr(positions), _ptr(seq_of_token), _ptr(slots), _ptr(block_table), block_table.shape[1] if block_table is not None else 0,
+             _ptr(cache), _ptr(q_plain), _ptr(q_wide), _is_bf16(q_plain, "latent_prepare"), T, H, D, DR, R, int(rot), page, _stream()),
+           "latent_prepare")
+
+
+# ---------------------------------------------------------------- routed experts -----
+def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch.Tensor, share: torch.Tensor, top: int) -> None:
+    """scores float [T, E] (+ bias [E]): the `top` largest per row (ties to the lower number) into chosen int32 [T, top],
+    the softmax over them into share float [T, top]."""
+    _dev("route_topk", scores, bias, chosen, share)
+    T, E = scores.shape
+    _req(scores.dtype == torch.float32 and (bias is None or (bias.dtype == torch.float32 and bias.numel() == E)), "route_topk: float32 scores and bias")
+    _req(chosen.dtype == torch.int32 and chosen.shape == (T, top) and share.dtype == torch.float32 and share.shape == (T, top), "route_topk: chosen int32 and share float32 [T, top]")
+    _req(0 < top <= min(E, 64) and E <= 512, f"route_topk: {top} of {E} experts is outside the kernel's sizes (512 experts, 64 chosen)")
+    f = _fn("routed_experts", "br_route_topk", [_P, _P, _P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(scores), _ptr(bias), _ptr(chosen), _ptr(share), T, E, top, _stream()), "route_topk")
+
+
+def experts_up(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, chosen: torch.Tensor, y: torch.Tensor) -> None:
+    """y[t, s] = silu(W_gate[e] h[t]) * (W_up[e] h[t]) with e = chosen[t, s]; weights [E, F, W], y [T, top, F]."""
+    _dev("experts_up", h, w_gate, w_up, chosen, y)
+    T, W = h.shape
+    E, F, _ = w_gate.shape
+    top = chosen.shape[1]
+    _req(w_gate.shape == w_up.shape == (E, F, W) and y.shape == (T, top, F) and chosen.shape == (T, top) and chosen.dtype == torch.int32, "experts_up: shapes")
+    _req(h.dtype == w_gate.dtype == w_up.dtype == y.dtype, "experts_up: one type for rows and weights")
+    _req(W <= 16384, "experts_up: rows wider than 16,384")
+    f = _fn("routed_experts", "br_experts_up", [_P, _P, _P, _P, _P] + [c_int] * 5 + [_P])
+    _check(f(_ptr(h), _ptr(w_gate), _ptr(w_up), _ptr(chosen), _ptr(y), _is_bf16(h, "experts_up"), T, W, F, top, _stream()), "experts_up")
+
+
+def experts_down(y: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, share: torch.Tensor, x: torch.Tensor) -> None:
+    """x[t] += sum_s share[t, s] * W_down[chosen[t, s]] y[t, s]; w_down [E, W, F], x float [T, W]."""
+    _dev("experts_down", y, w_down, chosen, share, x)
+    T, top, F = y.shape
+    E, W, _ = w_down.shape
+    _req(w_down.shape == (E, W, F) and x.shape == (T, W) and x.dtype == torch.float32 and chosen.shape == (T, top) and share.shape == (T, top), "experts_down: shapes")
+    _req(y.dtype == w_down.dtype and chosen.dtype == torch.int32 and share.dtype == torch.float32, "experts_down: types")
+    _req(top * F <= 16384, "experts_down: more than 16,384 inner elements a token")
+    f = _fn("routed_experts", "br_experts_down", [_P, _P, _P, _P, _P] + [c_int] * 5 + [_P])
+    _check(f(_ptr(y), _ptr(w_down), _ptr(chosen), _ptr(share), _ptr(x), _is_bf16(y, "experts_down"), T, W, F, top, _stream()), "experts_down")
+
+
+# ------------------------------------------------------------- clamped gated unit -----
+def clamped_glu(gu: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, limit: float, alpha: float) -> None:
+    """out = g sigmoid(alpha g) (u + 1), g = min(gate + b, limit), u = clamp(up + b, -limit, limit), from the float sums
+    gu [T, 2 I] (gate | up) and their biases [2 I]."""
+    _dev("clamped_glu", gu, bias, out)
+    T, I2 = gu.shape
+    _req(gu.dtype == torch.float32 and I2 % 2 == 0 and out.shape == (T, I2 // 2), "clamped_glu: gu float32 [T, 2 I], out [T, I]")
+    _req(bias is None or (bias.dtype == torch.float32 and bias.numel() == I2), "clamped_glu: bias float32 [2 I]")
+    f = _fn("elementwise", "br_clamped_glu", [_P, _P, _P, c_int, c_int, c_int, c_float, c_float, _P])
+    _check(f(_ptr(gu), _ptr(bias), _ptr(out), _is_bf16(out, "clamped_glu"), T, I2 // 2, float(limit), float(alpha), _stream()), "clamped_glu")
+
+
+def add_bias_rows(x: torch.Tensor, bias: torch.Tensor) -> None:
+    _dev("add_bias_rows", x, bias)
+    _req(x.dtype == torch.float32 and bias.dtype == torch.float32 and x.dim() == 2 and bias.numel() == x.shape[1], "add_bias_rows: x float32 [T, H], bias float32 [H]")
+    f = _fn("elementwise", "br_add_bias_rows", [_P, _P, c_int, c_int, _P])
+    _check(f(_ptr(x), _ptr(bias), x.shape[0], x.shape[1], _stream()), "add_bias_rows")
 
 
 def attention_prefill_bf16(q: torch.Tensor, q_stride: int, out: torch.Tensor, cu_seqlens: torch.Tensor,

@@ -4,6 +4,9 @@ x += feed_forward(norm(x)), with the layer's norms of the roles "mixer" and "fee
 compile_attention.rs:78-376, compile_layers.rs:373-386).  The parts add into `x`
 themselves, so the sum is part of their last projection.
 
+`sandwich_residual` norms a half's output too before the sum; `parallel_residual` runs both halves on one
+normed input, x += mixer(norm(x)) + feed_forward(norm(x)).
+
 An arrangement is an object with `run(layer, x, step, mixer_ctx)`; it reads whatever roles
 of `layer.norms` it likes.  It may also have `first_norm(layer)`: the norm that reads the
 residual rows first when the layer runs, which lets the layer before prepare that norm
@@ -112,5 +115,31 @@ class SandwichResidual:
             step.prepared_norm = (next_norm, x, ("normed", h_next))
 
 
+class ParallelResidual:
+    """x += mixer(n) + feed_forward(n) with n = norm(x): one norm (role "mixer") whose output both halves read.
+    Each half adds its output into the residual rows in its last product, the mixer first; neither reads the rows."""
+
+    def first_norm(self, layer):
+        return layer.norms.get("mixer")
+
+    def run(self, layer, x, step, mixer_ctx) -> None:
+        step.prepared_norm = None
+        dtype = layer.rt.dtype
+        norm = layer.norms.get("mixer")
+        h = x
+        if norm is not None:
+            h = step.ws.get("block_h", tuple(x.shape), dtype)
+            norm.forward(x, h)
+        if layer.mixer is not None:
+            layer.mixer.forward(h, x, step, mixer_ctx)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_mixer", x)
+        if layer.feed_forward is not None:
+            layer.feed_forward.forward(h, x, step)
+        if step.probe is not None:
+            step.probe(f"L{step.schedule_index}.post_ffn", x)
+
+
 register_part("block", "prenorm_residual", PrenormResidual, replace=True)
+register_part("block", "parallel_residual", ParallelResidual, replace=True)
 register_part("block", "sandwich_residual", SandwichResidual, replace=True)

@@ -1,6 +1,14 @@
 """SwiGLU feed-forward: x += W_d (silu(W_g n) * (W_u n)), silu(g) = g / (1 + exp(-g))
 (reference: op_ffn_gate_up_wx and op_ffn_down_res, kernels/megakernel_ops.hip:1474-1553,
-:1559-1602; the activation is fixed to SiLU there, :1538-1544)."""
+:1559-1602; the activation is fixed to SiLU there, :1538-1544).
+
+Clamped gated unit: with g = min(W_g n + b_g, limit) and u = clamp(W_u n + b_u, -limit, limit),
+x += W_d (g sigmoid(alpha g) (u + 1)) + b_d; every projection has a bias, the clamps and the activation work on
+the products' float sums.
+
+Routed experts: router scores z = W_r n + b_r in float; a token takes the `top` experts with the largest scores
+(ties to the lower number), weighted by the softmax over those scores only, and x += sum_s share_s expert_s(n)
+with an expert W_d (silu(W_g n) * (W_u n)) without biases.  The reference has neither."""
 from __future__ import annotations
 
 from typing import Dict, List, Optional
@@ -8,6 +16,7 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import kernels as K
+from ..errors import ConfigError
 from ..weights import TensorSpec
 from .base import FeedForward, NormedInput, Runtime, register_part
 from .linear import fused_layout, linear, stream_layout
@@ -62,4 +71,103 @@ class SwiGLU(FeedForward):
         linear(a, self.w_d, x, step.ws, accumulate=True)
 
 
+class ClampedGLU(FeedForward):
+    graph_safe = True
+
+    NAMES = {"gate": "gate", "gate_bias": "gate.b", "up": "up", "up_bias": "up.b", "down": "down", "down_bias": "down.b"}
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702,
+                 names: Optional[Dict[str, str]] = None):
+        self.H, self.I, self.limit, self.alpha = int(hidden_size), int(intermediate_size), float(limit), float(alpha)
+        if self.I <= 0 or not self.limit > 0:
+            raise ConfigError(f"clamped gated unit: an inner width of {intermediate_size} and a limit of {limit} must be positive")
+        self.names = dict(self.NAMES, **(names or {}))
+        self.w_gu = self.w_d = self.b_gu = self.b_d = None
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        n = self.names
+        return [TensorSpec(prefix + n["gate"], (self.I, self.H)),
+                TensorSpec(prefix + n["gate_bias"], (self.I,), kind="vector", init="normal"),
+                TensorSpec(prefix + n["up"], (self.I, self.H)),
+                TensorSpec(prefix + n["up_bias"], (self.I,), kind="vector", init="normal"),
+                TensorSpec(prefix + n["down"], (self.H, self.I)),
+                TensorSpec(prefix + n["down_bias"], (self.H,), kind="vector", init="normal")]
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        n = self.names
+        self.w_gu = fused_layout([tensors[prefix + n["gate"]], tensors[prefix + n["up"]]], rt)
+        self.w_d = stream_layout(tensors[prefix + n["down"]], rt)
+        self.b_gu = rt.own(torch.cat([tensors[prefix + n[x]].to(torch.float32).reshape(-1) for x in ("gate_bias", "up_bias")]))
+        self.b_d = rt.own(tensors[prefix + n["down_bias"]].to(torch.float32).reshape(-1))
+
+    def forward(self, h, x, step) -> None:
+        T = step.n_tokens
+        gu = step.ws.get("ffn_gu32", (T, 2 * self.I), torch.float32)
+        linear(h, self.w_gu, gu, step.ws)
+        a = step.ws.get("ffn_act", (T, self.I), self.rt.dtype)
+        K.clamped_glu(gu, self.b_gu, a, self.limit, self.alpha)
+        linear(a, self.w_d, x, step.ws, accumulate=True)
+        K.add_bias_rows(x, self.b_d)
+
+
+class RoutedExperts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, router_bias: bool = True,
+                 names: Optional[Dict[str, str]] = None):
+        """`names`: "expert" with {e} for the expert's number (the prefix of its three matrices "gate", "up", "down"),
+        "router", "router_bias"."""
+        self.H, self.I, self.E, self.top = int(hidden_size), int(intermediate_size), int(num_experts), int(top)
+        if self.I <= 0 or not 0 < self.top <= self.E or self.E > 512 or self.top > 64:
+            raise ConfigError(f"routed experts: {top} of {num_experts} experts of inner width {intermediate_size} "
+                              "(at most 512 experts, 64 chosen)")
+        self.router_bias = bool(router_bias)
+        self.names = dict({"expert": "e{e}.", "gate": "gate", "up": "up", "down": "down", "router": "router",
+                           "router_bias": "router.b"}, **(names or {}))
+        self.w_gate = self.w_up = self.w_down = self.w_router = self.b_router = None
+
+    def _expert(self, prefix: str, e: int, what: str) -> str:
+        return prefix + self.names["expert"].format(e=e) + self.names[what]
+
+    def weight_specs(self, prefix: str) -> List[TensorSpec]:
+        out = []
+        for e in range(self.E):
+            out += [TensorSpec(self._expert(prefix, e, "gate"), (self.I, self.H)),
+                    TensorSpec(self._expert(prefix, e, "up"), (self.I, self.H)),
+                    TensorSpec(self._expert(prefix, e, "down"), (self.H, self.I))]
+        out.append(TensorSpec(prefix + self.names["router"], (self.E, self.H)))
+        if self.router_bias:
+            out.append(TensorSpec(prefix + self.names["router_bias"], (self.E,), kind="vector", init="normal"))
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
+        self.rt = rt
+        first = tensors[self._expert(prefix, 0, "gate")]
+        # the experts' matrices stacked, so that a kernel finds expert e's rows by its number
+        self.w_gate = rt.empty((self.E, self.I, self.H), first.dtype)
+        self.w_up = rt.empty((self.E, self.I, self.H), first.dtype)
+        self.w_down = rt.empty((self.E, self.H, self.I), first.dtype)
+        for e in range(self.E):
+            self.w_gate[e].copy_(first if e == 0 else tensors[self._expert(prefix, e, "gate")])
+            self.w_up[e].copy_(tensors[self._expert(prefix, e, "up")])
+            self.w_down[e].copy_(tensors[self._expert(prefix, e, "down")])
+        self.w_router = rt.own(tensors[prefix + self.names["router"]])
+        if self.router_bias:
+            self.b_router = rt.own(tensors[prefix + self.names["router_bias"]].to(torch.float32).reshape(-1))
+
+    def forward(self, h, x, step) -> None:
+        T, dt = step.n_tokens, self.rt.dtype
+        scores = step.ws.get("moe_scores", (T, self.E), torch.float32)
+        linear(h, self.w_router, scores, step.ws)
+        chosen = step.ws.get("moe_chosen", (T, self.top), torch.int32)
+        share = step.ws.get("moe_share", (T, self.top), torch.float32)
+        K.route_topk(scores, self.b_router, chosen, share, self.top)
+        y = step.ws.get("moe_y", (T, self.top, self.I), dt)
+        K.experts_up(h, self.w_gate, self.w_up, chosen, y)
+        K.experts_down(y, self.w_down, chosen, share, x)
+
+
 register_part("feed_forward", "swiglu", SwiGLU, replace=True)
+register_part("feed_forward", "clamped_glu", ClampedGLU, replace=True)
+register_part("feed_forward", "routed_experts", RoutedExperts, replace=True)

@@ -6,10 +6,18 @@ inv_freq[p] = 1 / theta^(2p / rotary_dim) in float32 and theta = float(pos) * in
 kernels/megakernel_ops.hip:2019-2024).  `pairing` says which elements form a pair:
 "adjacent" (2p, 2p+1) as the reference's kernel does (:2025-2030), or "half"
 (p, p + rotary_dim/2), the layout of MistralForCausalLM checkpoints.
+
+`scaling` = {factor, original, fast, slow} stretches the encoding beyond the `original` positions a model was
+made for: with i(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta) the (real-valued) pair whose
+wavelength makes t turns over `original` positions, lo = max(floor(i(fast)), 0), hi = min(ceil(i(slow)),
+rotary_dim - 1) and ramp_p = clamp((p - lo) / max(hi - lo, 0.001), 0, 1), pair p turns with
+inv_freq[p] / factor * ramp_p + inv_freq[p] * (1 - ramp_p) (fast pairs keep their frequency, slow ones are
+slowed by `factor`), and cos and sin are multiplied by 0.1 ln(factor) + 1.  The reference has no such scaling.
 """
 from __future__ import annotations
 
-from typing import Dict
+import math
+from typing import Dict, Optional
 
 import torch
 
@@ -22,18 +30,49 @@ class RotaryEncoding(PositionEncoding):
     graph_safe = True
     gives = "rotary"
 
-    def __init__(self, rotary_dim: int, theta: float, pairing: str = "half"):
+    def __init__(self, rotary_dim: int, theta: float, pairing: str = "half", scaling: Optional[Dict[str, float]] = None):
         if rotary_dim <= 0 or rotary_dim % 2:
             raise ConfigError(f"rotary_dim must be positive and even, got {rotary_dim}")
         if pairing not in ("half", "adjacent"):
             raise ConfigError(f"rope pairing must be 'half' or 'adjacent', got {pairing!r}")
         self.rotary_dim, self.theta, self.pairing = int(rotary_dim), float(theta), pairing
+        self.scaling = None
+        self.magnitude = 1.0
+        if scaling is not None:
+            try:
+                self.scaling = {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
+            except (KeyError, TypeError, ValueError):
+                raise ConfigError(f"rope scaling needs the numbers factor, original, fast and slow, got {scaling!r}") from None
+            if min(self.scaling.values()) <= 0 or self.theta <= 1.0:
+                raise ConfigError(f"rope scaling takes positive numbers and a base above 1, got {scaling!r} with base {theta}")
+            self.magnitude = 0.1 * math.log(self.scaling["factor"]) + 1.0
         self.inv_freq = None
+
+    def frequencies(self):
+        """The pairs' frequencies as Python floats (float64 arithmetic; the device keeps their float32 roundings)."""
+        n, half = self.rotary_dim, self.rotary_dim // 2
+        f = [self.theta ** (-2.0 * p / n) for p in range(half)]
+        sc = self.scaling
+        if sc is None:
+            return f
+
+        def pair_of(turns):
+            return n * math.log(sc["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+        lo = max(math.floor(pair_of(sc["fast"])), 0)
+        hi = min(math.ceil(pair_of(sc["slow"])), n - 1)
+        out = []
+        for p in range(half):
+            ramp = min(max((p - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(f[p] / sc["factor"] * ramp + f[p] * (1.0 - ramp))
+        return out
 
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
-        expo = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / float(self.rotary_dim)
-        inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32), expo)
+        if self.scaling is None:
+            expo = torch.arange(0, self.rotary_dim, 2, dtype=torch.float32) / float(self.rotary_dim)
+            inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float32), expo)
+        else:
+            inv = torch.tensor(self.frequencies(), dtype=torch.float64)
         self.inv_freq = inv.to(torch.float32).to(rt.device)
 
     def prepare(self, step) -> RotaryTables:
@@ -43,6 +82,9 @@ class RotaryEncoding(PositionEncoding):
         cos = step.ws.get(f"rope_cos_{id(self)}", (step.n_tokens, P), torch.float32)
         sin = step.ws.get(f"rope_sin_{id(self)}", (step.n_tokens, P), torch.float32)
         K.rope_table(step.position_ids, self.inv_freq, cos, sin)
+        if self.magnitude != 1.0:
+            K.scale_(cos, self.magnitude)
+            K.scale_(sin, self.magnitude)
         return RotaryTables(cos, sin, self.rotary_dim, self.pairing == "adjacent")
 
 
