@@ -348,9 +348,12 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(
     const int cg = lane >> 4, g = lane & 15;
     const int cb4 = cb16 * 4 + wave, c = cb4 * 4 + cg;
     const int slot = slots[s];
-    if (slot < 0) return;
     const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
     const bool live = c < e;
+    if (slot < 0) {                                // padding: no state behind it; its rows of o are zero
+        if (g == 0 && live) for (int t = t0; t < t1; ++t) o[(size_t)t * H * e + h * e + c] = 0.f;
+        return;
+    }
     const int ncb4 = (e + 3) >> 2;
     float* S = state + (size_t)slot * slot_stride + (((size_t)h * ncb4 + cb4) * RPL) * 64 + lane;
     float st[RPL], ub[RPL];

@@ -38,6 +38,7 @@ __global__ __launch_bounds__(64) void route_topk_kernel(const float* __restrict_
             const int oa = __shfl_xor(at, o, WAVE);
             if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
         }
+        if (at >= E) { at = s; best = first; }    // scores that compare with nothing (a padding row's): any expert will do
         if (s == 0) first = best;                 // the largest score: the softmax's shift
         const float w = expf(best - first);
         total += w;
