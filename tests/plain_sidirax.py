@@ -150,11 +150,15 @@ def clamped_glu_ff(h, w, p, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T + w[p + "down.b"]
 
 
-def routed_ff(h, w, p, experts, top):
+def routed_ff(h, w, p, experts, top, margins=None):
     """Every token through its `top` experts with the largest router logits, weighted by the softmax over those
-    logits only; an expert is W_d (silu(W_g h) * (W_u h))."""
+    logits only; an expert is W_d (silu(W_g h) * (W_u h)).  `margins` (a list) receives per token the distance
+    between the last chosen logit and the first one left out (how close the choice was)."""
     z = h @ w[p + "router"].T + w[p + "router.b"]
     out = np.zeros_like(h)
+    if margins is not None:
+        srt = -np.sort(-z, axis=1)
+        margins.append(srt[:, top - 1] - srt[:, top] if top < experts else np.full(h.shape[0], np.inf))
     for t in range(h.shape[0]):
         chosen = np.argsort(-z[t], kind="stable")[:top]
         a = np.exp(z[t, chosen] - z[t, chosen].max())
@@ -165,17 +169,18 @@ def routed_ff(h, w, p, experts, top):
     return out
 
 
-def feed_forward(h, w, p, mlp):
+def feed_forward(h, w, p, mlp, margins=None):
     if mlp is None:
         return np.zeros_like(h)
     if mlp["kind"] == "dense":
         return clamped_glu_ff(h, w, p, float(mlp["limit"]))
-    return routed_ff(h, w, p, mlp["router"]["experts"], mlp["router"]["top"])
+    return routed_ff(h, w, p, mlp["router"]["experts"], mlp["router"]["top"], margins)
 
 
 # ------------------------------------------------------------------ the model -------
-def forward(cfg, w, tokens, return_layers=False):
-    """Logits [T, vocab] of one sequence from position 0 (and the residual rows after every layer)."""
+def forward(cfg, w, tokens, return_layers=False, margins=None):
+    """Logits [T, vocab] of one sequence from position 0 (and the residual rows after every layer).  `margins` (a
+    list) receives one array per layer of routed experts, see `routed_ff`."""
     eps = float(cfg["norm"]["eps"])
     x = w["embed"][np.asarray(tokens)]
     kept, layers = {}, []
@@ -189,7 +194,7 @@ def forward(cfg, w, tokens, return_layers=False):
             mixed, rows = latent_attention_mixer(h, w, p + "mix.", m, eps, None if src is None else kept[src])
             if src is None:
                 kept[i] = rows
-        x = x + (mixed + feed_forward(h, w, p + "mlp.", l.get("mlp")))
+        x = x + (mixed + feed_forward(h, w, p + "mlp.", l.get("mlp"), margins))
         layers.append(x.copy())
     logits = rms_norm(x, w["final.norm"], eps) @ w["embed"].T
     return (logits, np.stack(layers)) if return_layers else logits
@@ -274,10 +279,10 @@ def random_weights(cfg, seed, gain=1.0):
         q = p + "mix."
         if l["type"] == "latent_attention":
             dr, e, r, qr = m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
-            w[q + "dq"], w[q + "dq.norm"], w[q + "uq"] = mat(qr, W), vec(qr), mat(H * (d + dr), qr, 2.0 * gain)
+            w[q + "dq"], w[q + "dq.norm"], w[q + "uq"] = mat(qr, W), vec(qr), mat(H * (d + dr), qr)
             if m.get("kv_from") is None:
                 w[q + "dkv"], w[q + "dkv.norm"] = mat(r + dr, W), vec(r)
-            w[q + "uk"], w[q + "uv"] = mat(H * d, r, 2.0 * gain), mat(H * e, r)
+            w[q + "uk"], w[q + "uv"] = mat(H * d, r), mat(H * e, r)
             w[q + "sink"] = vec(H, 0.5, 1.0)
             w[q + "o"] = mat(W, H * e)
         else:
