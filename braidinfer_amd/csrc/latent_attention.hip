@@ -3,8 +3,8 @@
 // value W_uv c, so with the query's unrotated part taken through W_uk^T first,
 //     score = (W_uk^T q_u) . c + q_r . k_r,        output = W_uv (sum_j p_j c_j),
 // which is attention of all heads over ONE row per token: keys [c | k_r] (R + DR wide), values c (R wide).
-// The products with W_uk^T and W_uv are the library's matrix products head by head, the attention itself is
-// the kernels of `pooled_attention.hip` with one kv head; this file prepares their operands.
+// The attention itself is the kernels of `pooled_attention.hip` with one kv head; this file prepares their
+// operands (`prepare`) and multiplies head by head (`head_linear`: the products with W_uk^T and W_uv).
 //
 // `prepare`, a workgroup per token:
 //   * c = rms_norm(dkv[0:R]) * weight and k_r = rotate(dkv[R:R+DR]) into the token's cache page: the key row
@@ -88,5 +88,78 @@ extern "C" int br_latent_prepare(const float* q, size_t q_stride, const float* d
         slots, block_table, table_stride, (bf16*)cache, (bf16*)q_plain, (bf16*)q_wide, H, D, DR, R, rot, page);
     else latent_prepare_kernel<float><<<T, 256, 0, s>>>(q, q_stride, dkv, dkv_stride, c_weight, eps, cs, sn, pos, seq_of_token,
         slots, block_table, table_stride, (float*)cache, (float*)q_plain, (float*)q_wide, H, D, DR, R, rot, page);
+    return br_check_launch();
+}
+
+// ------------------------------------------------------- a product head by head -----
+// out[t, h, n] = sum_k a[t, h, k] * w[h, n, k]: every head's rows through a matrix of its own, all heads in one
+// launch (the products with W_uk^T and W_uv around the attention).  a and out are [T, H, .] views: rows `lda` /
+// `ldo` elements apart, heads `a_hs` / `o_hs` apart; w is [H, N, K] dense.
+//
+// bfloat16 on the matrix cores: a wave owns 32 outputs n x 32 tokens t and walks k 16 at a time with
+// v_mfma_f32_32x32x16_bf16, the weight rows as the first operand (so a lane ends with four neighbouring n of one
+// token in four neighbouring registers), both operands straight from memory 16 bytes a lane; four waves a
+// workgroup side by side along n.  grid (ceil(T / 32), ceil(N / 128), H).  K in steps of 8, rows and heads of a
+// at multiples of 16 bytes.
+__global__ __launch_bounds__(256) void head_linear_bf16_kernel(const bf16* __restrict__ a, size_t lda, size_t a_hs,
+                                                               const bf16* __restrict__ w, bf16* __restrict__ out, size_t ldo,
+                                                               size_t o_hs, int T, int N, int K) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, g = lane >> 5;
+    const int t0 = blockIdx.x * 32, n0 = blockIdx.y * 128 + wave * 32, h = blockIdx.z;
+    if (n0 >= N) return;
+    const int t = t0 + c, nrow = n0 + c;
+    const bf16* wrow = w + ((size_t)h * N + (nrow < N ? nrow : N - 1)) * K;
+    const bf16* arow = a + (size_t)(t < T ? t : T - 1) * lda + (size_t)h * a_hs;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    bf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        const int k = k0 + 8 * g;
+        const bf16x8 wf = (k < K && nrow < N) ? *(const bf16x8*)(wrow + k) : zero;
+        const bf16x8 af = (k < K && t < T) ? *(const bf16x8*)(arow + k) : zero;
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, af, acc, 0, 0, 0);
+    }
+    if (t >= T) return;
+    bf16* orow = out + (size_t)t * ldo + (size_t)h * o_hs;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int n = n0 + 8 * (r >> 2) + 4 * g + (r & 3);
+        if (n < N) orow[n] = (bf16)acc[r];
+    }
+}
+
+// Any type and alignment: a thread an output, float sums in ascending k.
+template <typename T>
+__global__ __launch_bounds__(256) void head_linear_plain_kernel(const T* __restrict__ a, size_t lda, size_t a_hs,
+                                                                const T* __restrict__ w, T* __restrict__ out, size_t ldo,
+                                                                size_t o_hs, int n_tok, int H, int N, int K) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)n_tok * H * N) return;
+    const int n = (int)(i % N), h = (int)((i / N) % H);
+    const size_t t = i / ((size_t)N * H);
+    const T* ar = a + t * lda + (size_t)h * a_hs;
+    const T* wr = w + ((size_t)h * N + n) * K;
+    float s = 0.f;
+    for (int k = 0; k < K; ++k) s = fmaf(to_f32<T>(ar[k]), to_f32<T>(wr[k]), s);
+    out[t * ldo + (size_t)h * o_hs + n] = from_f32<T>(s);
+}
+
+extern "C" int br_head_linear(const void* a, size_t lda, size_t a_hs, const void* w, void* out, size_t ldo, size_t o_hs,
+                              int is_bf16, int T, int H, int N, int K, hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (H <= 0 || N <= 0 || K <= 0 || H > 65535 || (N + 127) / 128 > 65535) return BR_BAD_ARG;
+    if (is_bf16 && K % 8 == 0 && lda % 8 == 0 && a_hs % 8 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0) {
+        dim3 grid((T + 31) / 32, (N + 127) / 128, H);
+        head_linear_bf16_kernel<<<grid, 256, 0, s>>>((const bf16*)a, lda, a_hs, (const bf16*)w, (bf16*)out, ldo, o_hs, T, N, K);
+        return br_check_launch();
+    }
+    const size_t n = (size_t)T * H * N;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (is_bf16) head_linear_plain_kernel<bf16><<<blocks, 256, 0, s>>>((const bf16*)a, lda, a_hs, (const bf16*)w, (bf16*)out, ldo, o_hs, T, H, N, K);
+    else head_linear_plain_kernel<float><<<blocks, 256, 0, s>>>((const float*)a, lda, a_hs, (const float*)w, (float*)out, ldo, o_hs, T, H, N, K);
     return br_check_launch();
 }

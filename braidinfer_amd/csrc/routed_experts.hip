@@ -1,14 +1,16 @@
 // A feed-forward of routed experts: every token goes through the `top` experts with the largest router
 // scores and takes their outputs weighted by the softmax over those scores only.  An expert is
-// W_d (silu(W_g h) * (W_u h)) without biases; the experts' matrices lie stacked, [E][F][W] for gate and up and
-// [E][W][F] for down.
+// W_d (silu(W_g h) * (W_u h)) without biases; the experts' matrices lie stacked, [E][2 F][W] for gate (an expert's
+// first F rows) and up (its last F) and [E][W][F] for down.
 //
 //   route:  scores (the router product's float sums) + bias -> the chosen experts and their shares, float;
 //           ties go to the lower expert number.
 //   up:     y[t, s, :] = silu(W_g[e] h_t) * (W_u[e] h_t) for slot s of token t with e its expert.
 //   down:   x[t, :] += sum_s share[t, s] * W_d[e_s] y[t, s, :], slots added in slot order in float.
 // `up` and `down` read an expert's rows once per (token, slot): the form for steps of few tokens, where the
-// experts' weights are what a step reads.
+// experts' weights are what a step reads.  Steps of many tokens go expert by expert through the library's matrix
+// products instead: `sort` groups the (token, slot) pairs by expert, `gather` copies their rows into that order,
+// and `combine` adds every token's weighted outputs back in slot order.
 #include "common.h"
 
 #define RX_MAX_PER_LANE 8          // experts a lane keeps: up to 512 experts
@@ -83,17 +85,16 @@ __device__ __forceinline__ float rx_dot(const T* __restrict__ wrow, const float*
 
 // grid (T * top, ceil(F / 16)), 4 waves, a wave four columns.  LDS: W floats.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void experts_up_kernel(const T* __restrict__ h, const T* __restrict__ w_gate,
-                                                         const T* __restrict__ w_up, const int* __restrict__ chosen,
-                                                         T* __restrict__ y, int W, int F, int top) {
+__global__ __launch_bounds__(256) void experts_up_kernel(const T* __restrict__ h, const T* __restrict__ w_gu,
+                                                         const int* __restrict__ chosen, T* __restrict__ y, int W, int F, int top) {
     extern __shared__ float hs[];
     const int slot = blockIdx.x, t = slot / top;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < W; i += 256) hs[i] = to_f32<T>(h[(size_t)t * W + i]);
     __syncthreads();
     const int e = chosen[slot];
-    const T* wg = w_gate + (size_t)e * F * W;
-    const T* wu = w_up + (size_t)e * F * W;
+    const T* wg = w_gu + (size_t)e * 2 * F * W;
+    const T* wu = wg + (size_t)F * W;
     for (int j = 0; j < 4; ++j) {
         const int f = blockIdx.y * 16 + wave * 4 + j;
         if (f >= F) break;
@@ -126,14 +127,14 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
     }
 }
 
-extern "C" int br_experts_up(const void* h, const void* w_gate, const void* w_up, const int* chosen, void* y, int is_bf16,
+extern "C" int br_experts_up(const void* h, const void* w_gu, const int* chosen, void* y, int is_bf16,
                              int T, int W, int F, int top, hipStream_t s) {
     if (T <= 0) return BR_OK;
     if (W <= 0 || F <= 0 || top <= 0 || (size_t)W * 4 > 65536 || (F + 15) / 16 > 65535) return BR_BAD_ARG;
     dim3 grid((unsigned)((size_t)T * top), (F + 15) / 16);
     const size_t lds = (size_t)W * sizeof(float);
     const bool vec = W % (is_bf16 ? 8 : 4) == 0;
-#define RX_UP(TT, V) experts_up_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)h, (const TT*)w_gate, (const TT*)w_up, chosen, (TT*)y, W, F, top)
+#define RX_UP(TT, V) experts_up_kernel<TT, V><<<grid, 256, lds, s>>>((const TT*)h, (const TT*)w_gu, chosen, (TT*)y, W, F, top)
     if (is_bf16) { if (vec) RX_UP(bf16, true); else RX_UP(bf16, false); }
     else { if (vec) RX_UP(float, true); else RX_UP(float, false); }
 #undef RX_UP
@@ -151,5 +152,75 @@ extern "C" int br_experts_down(const void* y, const void* w_down, const int* cho
     if (is_bf16) { if (vec) RX_DOWN(bf16, true); else RX_DOWN(bf16, false); }
     else { if (vec) RX_DOWN(float, true); else RX_DOWN(float, false); }
 #undef RX_DOWN
+    return br_check_launch();
+}
+
+// ------------------------------------------------------------ expert by expert -----
+// The (token, slot) pairs grouped by expert: first[e] .. first[e + 1] - 1 are the places of expert e's pairs in
+// `order` (pair numbers t * top + s), and place[pair] is where a pair went.  One workgroup: counts in LDS, a scan by
+// one thread, places handed out by counters.  Which of an expert's pairs comes first is left to the counters; a
+// pair's output does not depend on its place.
+__global__ __launch_bounds__(1024) void experts_sort_kernel(const int* __restrict__ chosen, int* __restrict__ first,
+                                                            int* __restrict__ order, int* __restrict__ place, int n, int E) {
+    extern __shared__ int cnt[];                   // [E] counts, then [E] counters
+    int* cur = cnt + E;
+    for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) atomicAdd(&cnt[chosen[i]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int e = 0; e < E; ++e) { first[e] = at; cur[e] = at; at += cnt[e]; }
+        first[E] = at;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const int p = atomicAdd(&cur[chosen[i]], 1);
+        order[p] = i;
+        place[i] = p;
+    }
+}
+
+extern "C" int br_experts_sort(const int* chosen, int* first, int* order, int* place, int n, int E, hipStream_t s) {
+    if (n <= 0) return BR_OK;
+    if (E <= 0 || E > 4096) return BR_BAD_ARG;
+    experts_sort_kernel<<<1, 1024, 2 * E * sizeof(int), s>>>(chosen, first, order, place, n, E);
+    return br_check_launch();
+}
+
+// rows[p, :] = h[order[p] / top, :]: the tokens' rows in the experts' order.  grid (pairs), 256 threads.
+template <typename T>
+__global__ __launch_bounds__(256) void experts_gather_kernel(const T* __restrict__ h, const int* __restrict__ order,
+                                                             T* __restrict__ rows, int W, int top) {
+    const T* src = h + (size_t)(order[blockIdx.x] / top) * W;
+    T* dst = rows + (size_t)blockIdx.x * W;
+    for (int i = threadIdx.x; i < W; i += 256) dst[i] = src[i];
+}
+
+extern "C" int br_experts_gather(const void* h, const int* order, void* rows, int is_bf16, int n, int W, int top, hipStream_t s) {
+    if (n <= 0) return BR_OK;
+    if (W <= 0 || top <= 0) return BR_BAD_ARG;
+    if (is_bf16) experts_gather_kernel<bf16><<<n, 256, 0, s>>>((const bf16*)h, order, (bf16*)rows, W, top);
+    else experts_gather_kernel<float><<<n, 256, 0, s>>>((const float*)h, order, (float*)rows, W, top);
+    return br_check_launch();
+}
+
+// x[t, :] += sum_s share[t, s] * out[place[t * top + s], :] with out the experts' float outputs in their order;
+// slots in slot order.  grid (T, ceil(W / 256)).
+__global__ __launch_bounds__(256) void experts_combine_kernel(const float* __restrict__ out, const int* __restrict__ place,
+                                                              const float* __restrict__ share, float* __restrict__ x, int W, int top) {
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    if (i >= W) return;
+    float sum = 0.f;
+    for (int s = 0; s < top; ++s)
+        sum = fmaf(share[(size_t)t * top + s], out[(size_t)place[(size_t)t * top + s] * W + i], sum);
+    x[(size_t)t * W + i] += sum;
+}
+
+extern "C" int br_experts_combine(const float* out, const int* place, const float* share, float* x, int T, int W, int top,
+                                  hipStream_t s) {
+    if (T <= 0) return BR_OK;
+    if (W <= 0 || top <= 0 || (W + 255) / 256 > 65535) return BR_BAD_ARG;
+    experts_combine_kernel<<<dim3(T, (W + 255) / 256), 256, 0, s>>>(out, place, share, x, W, top);
     return br_check_launch();
 }

@@ -835,6 +835,20 @@ def latent_prepare(q: torch.Tensor, dkv: Optional[torch.Tensor], c_weight: Optio
            "latent_prepare")
 
 
+def head_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, h, :] = w[h] a[t, h, :] for every head in one launch: a [T, H, K] and out [T, H, N] may be views of
+    wider rows (strides between tokens and heads, dense last dimension); w [H, N, K] dense."""
+    _dev("head_linear", w)
+    T, H, K = a.shape
+    N = w.shape[1]
+    _req(a.is_cuda and out.is_cuda and a.dtype == w.dtype == out.dtype, "head_linear: one type, on the device")
+    _req(w.shape == (H, N, K) and out.shape == (T, H, N) and a.stride(2) == 1 and out.stride(2) == 1, "head_linear: a [T, H, K], w [H, N, K], out [T, H, N]")
+    lda, ldo = (a.stride(0) if T > 1 else H * K), (out.stride(0) if T > 1 else H * N)
+    f = _fn("latent_attention", "br_head_linear", [_P, c_size_t, c_size_t, _P, _P, c_size_t, c_size_t] + [c_int] * 5 + [_P])
+    _check(f(_ptr(a), lda, a.stride(1) if H > 1 else K, _ptr(w), _ptr(out), ldo, out.stride(1) if H > 1 else N, _is_bf16(a, "head_linear"),
+             T, H, N, K, _stream()), "head_linear")
+
+
 # ---------------------------------------------------------------- routed experts -----
 def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch.Tensor, share: torch.Tensor, top: int) -> None:
     """scores float [T, E] (+ bias [E]): the `top` largest per row (ties to the lower number) into chosen int32 [T, top],
@@ -848,17 +862,48 @@ def route_topk(scores: torch.Tensor, bias: Optional[torch.Tensor], chosen: torch
     _check(f(_ptr(scores), _ptr(bias), _ptr(chosen), _ptr(share), T, E, top, _stream()), "route_topk")
 
 
-def experts_up(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, chosen: torch.Tensor, y: torch.Tensor) -> None:
-    """y[t, s] = silu(W_gate[e] h[t]) * (W_up[e] h[t]) with e = chosen[t, s]; weights [E, F, W], y [T, top, F]."""
-    _dev("experts_up", h, w_gate, w_up, chosen, y)
+def experts_up(h: torch.Tensor, w_gu: torch.Tensor, chosen: torch.Tensor, y: torch.Tensor) -> None:
+    """y[t, s] = silu(W_gate[e] h[t]) * (W_up[e] h[t]) with e = chosen[t, s]; w_gu [E, 2 F, W] holds an expert's gate
+    rows, then its up rows; y [T, top, F]."""
+    _dev("experts_up", h, w_gu, chosen, y)
     T, W = h.shape
-    E, F, _ = w_gate.shape
+    E, F2, _ = w_gu.shape
     top = chosen.shape[1]
-    _req(w_gate.shape == w_up.shape == (E, F, W) and y.shape == (T, top, F) and chosen.shape == (T, top) and chosen.dtype == torch.int32, "experts_up: shapes")
-    _req(h.dtype == w_gate.dtype == w_up.dtype == y.dtype, "experts_up: one type for rows and weights")
+    _req(F2 % 2 == 0 and w_gu.shape == (E, F2, W) and y.shape == (T, top, F2 // 2) and chosen.shape == (T, top) and chosen.dtype == torch.int32, "experts_up: shapes")
+    _req(h.dtype == w_gu.dtype == y.dtype, "experts_up: one type for rows and weights")
     _req(W <= 16384, "experts_up: rows wider than 16,384")
-    f = _fn("routed_experts", "br_experts_up", [_P, _P, _P, _P, _P] + [c_int] * 5 + [_P])
-    _check(f(_ptr(h), _ptr(w_gate), _ptr(w_up), _ptr(chosen), _ptr(y), _is_bf16(h, "experts_up"), T, W, F, top, _stream()), "experts_up")
+    f = _fn("routed_experts", "br_experts_up", [_P, _P, _P, _P] + [c_int] * 5 + [_P])
+    _check(f(_ptr(h), _ptr(w_gu), _ptr(chosen), _ptr(y), _is_bf16(h, "experts_up"), T, W, F2 // 2, top, _stream()), "experts_up")
+
+
+def experts_sort(chosen: torch.Tensor, first: torch.Tensor, order: torch.Tensor, place: torch.Tensor, E: int) -> None:
+    """The (token, slot) pairs of chosen [T, top] grouped by expert: first int32 [E + 1], order and place int32 [T * top]."""
+    _dev("experts_sort", chosen, first, order, place)
+    n = chosen.numel()
+    _req(chosen.dtype == first.dtype == order.dtype == place.dtype == torch.int32 and first.numel() == E + 1 and order.numel() == n
+         and place.numel() == n, "experts_sort: int32 arrays [E + 1], [pairs], [pairs]")
+    f = _fn("routed_experts", "br_experts_sort", [_P, _P, _P, _P, c_int, c_int, _P])
+    _check(f(_ptr(chosen), _ptr(first), _ptr(order), _ptr(place), n, E, _stream()), "experts_sort")
+
+
+def experts_gather(h: torch.Tensor, order: torch.Tensor, rows: torch.Tensor, top: int) -> None:
+    """rows[p] = h[order[p] // top]."""
+    _dev("experts_gather", h, order, rows)
+    n, W = rows.shape
+    _req(h.dtype == rows.dtype and h.shape[1] == W and order.dtype == torch.int32 and order.numel() == n, "experts_gather: shapes")
+    f = _fn("routed_experts", "br_experts_gather", [_P, _P, _P, c_int, c_int, c_int, c_int, _P])
+    _check(f(_ptr(h), _ptr(order), _ptr(rows), _is_bf16(h, "experts_gather"), n, W, top, _stream()), "experts_gather")
+
+
+def experts_combine(out: torch.Tensor, place: torch.Tensor, share: torch.Tensor, x: torch.Tensor) -> None:
+    """x[t] += sum_s share[t, s] * out[place[t * top + s]]; out float [T * top, W]."""
+    _dev("experts_combine", out, place, share, x)
+    T, top = share.shape
+    W = x.shape[1]
+    _req(out.dtype == x.dtype == share.dtype == torch.float32 and place.dtype == torch.int32 and out.shape == (T * top, W)
+         and x.shape == (T, W) and place.numel() == T * top, "experts_combine: shapes")
+    f = _fn("routed_experts", "br_experts_combine", [_P, _P, _P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(out), _ptr(place), _ptr(share), _ptr(x), T, W, top, _stream()), "experts_combine")
 
 
 def experts_down(y: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, share: torch.Tensor, x: torch.Tensor) -> None:

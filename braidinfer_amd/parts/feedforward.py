@@ -125,7 +125,7 @@ class RoutedExperts(FeedForward):
         self.router_bias = bool(router_bias)
         self.names = dict({"expert": "e{e}.", "gate": "gate", "up": "up", "down": "down", "router": "router",
                            "router_bias": "router.b"}, **(names or {}))
-        self.w_gate = self.w_up = self.w_down = self.w_router = self.b_router = None
+        self.w_gu = self.w_down = self.w_router = self.b_router = None
 
     def _expert(self, prefix: str, e: int, what: str) -> str:
         return prefix + self.names["expert"].format(e=e) + self.names[what]
@@ -144,17 +144,20 @@ class RoutedExperts(FeedForward):
     def load(self, tensors: Dict[str, torch.Tensor], prefix: str, rt: Runtime) -> None:
         self.rt = rt
         first = tensors[self._expert(prefix, 0, "gate")]
-        # the experts' matrices stacked, so that a kernel finds expert e's rows by its number
-        self.w_gate = rt.empty((self.E, self.I, self.H), first.dtype)
-        self.w_up = rt.empty((self.E, self.I, self.H), first.dtype)
+        # the experts' matrices stacked, so that a kernel finds expert e's rows by its number: gate rows, then up rows
+        self.w_gu = rt.empty((self.E, 2 * self.I, self.H), first.dtype)
         self.w_down = rt.empty((self.E, self.H, self.I), first.dtype)
         for e in range(self.E):
-            self.w_gate[e].copy_(first if e == 0 else tensors[self._expert(prefix, e, "gate")])
-            self.w_up[e].copy_(tensors[self._expert(prefix, e, "up")])
+            self.w_gu[e, :self.I].copy_(first if e == 0 else tensors[self._expert(prefix, e, "gate")])
+            self.w_gu[e, self.I:].copy_(tensors[self._expert(prefix, e, "up")])
             self.w_down[e].copy_(tensors[self._expert(prefix, e, "down")])
         self.w_router = rt.own(tensors[prefix + self.names["router"]])
         if self.router_bias:
             self.b_router = rt.own(tensors[prefix + self.names["router_bias"]].to(torch.float32).reshape(-1))
+
+    # from this many tokens a step goes expert by expert through the matrix products (below it, every (token, slot)
+    # pair reads its expert's rows itself, which is what a step of few tokens costs anyway)
+    BY_EXPERT_FROM = 48
 
     def forward(self, h, x, step) -> None:
         T, dt = step.n_tokens, self.rt.dtype
@@ -163,9 +166,30 @@ class RoutedExperts(FeedForward):
         chosen = step.ws.get("moe_chosen", (T, self.top), torch.int32)
         share = step.ws.get("moe_share", (T, self.top), torch.float32)
         K.route_topk(scores, self.b_router, chosen, share, self.top)
-        y = step.ws.get("moe_y", (T, self.top, self.I), dt)
-        K.experts_up(h, self.w_gate, self.w_up, chosen, y)
-        K.experts_down(y, self.w_down, chosen, share, x)
+        if step.is_decode or T < self.BY_EXPERT_FROM:
+            y = step.ws.get("moe_y", (T, self.top, self.I), dt)
+            K.experts_up(h, self.w_gu, chosen, y)
+            K.experts_down(y, self.w_down, chosen, share, x)
+            return
+        # expert by expert: the pairs sorted by expert on the device, the experts' row counts read by the host
+        n = T * self.top
+        first = step.ws.get("moe_first", (self.E + 1,), torch.int32)
+        order = step.ws.get("moe_order", (n,), torch.int32)
+        place = step.ws.get("moe_place", (n,), torch.int32)
+        K.experts_sort(chosen, first, order, place, self.E)
+        rows = step.ws.get("moe_rows", (n, self.H), dt)
+        K.experts_gather(h, order, rows, self.top)
+        starts = first.tolist()
+        gu = step.ws.get("moe_gu", (n, 2 * self.I), dt)
+        act = step.ws.get("moe_act", (n, self.I), dt)
+        out = step.ws.get("moe_out", (n, self.H), torch.float32)
+        for e in range(self.E):
+            a, b = starts[e], starts[e + 1]
+            if b > a:
+                linear(rows[a:b], self.w_gu[e], gu[a:b], step.ws)
+                K.silu_mul(gu[a:b], act[a:b])
+                linear(act[a:b], self.w_down[e], out[a:b], step.ws)
+        K.experts_combine(out, place, share, x)
 
 
 register_part("feed_forward", "swiglu", SwiGLU, replace=True)

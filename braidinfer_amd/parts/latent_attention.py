@@ -148,8 +148,7 @@ class LatentAttention(Mixer):
                          step.positions, step.seq_of_token, step.slots, ctx.block_table, unit if self.own_rows else None,
                          q_plain, q_wide, nh, d, dr, r, ctx.page_tokens)
         # every head's plain part through its W_uk^T into the first kv_rank elements of its wide query
-        for hh in range(nh):
-            linear(q_plain[:, hh * d:(hh + 1) * d], self.w_uk_t[hh], q_wide[:, hh * wide:hh * wide + r], step.ws)
+        K.head_linear(q_plain.view(T, nh, d), self.w_uk_t, q_wide.view(T, nh, wide)[:, :, :r])
         o_lat = step.ws.get("la_o_lat", (T, nh * r), dt)
         sinks = self.sinks if self.sink else None
         if not step.is_decode and not self.force_simple and K.pwa_prefill_takes(dt, wide, r, ctx.page_tokens):
@@ -163,8 +162,7 @@ class LatentAttention(Mixer):
                          nh, 1, wide, r, ctx.page_tokens, NO_WINDOW, 0, self.scale, self.sink, sinks)
         # and every head's mixed latent through its W_uv
         o = step.ws.get("la_o", (T, nh * e), dt)
-        for hh in range(nh):
-            linear(o_lat[:, hh * r:(hh + 1) * r], self.w_uv[hh], o[:, hh * e:(hh + 1) * e], step.ws)
+        K.head_linear(o_lat.view(T, nh, r), self.w_uv, o.view(T, nh, e))
         linear(o, self.w_o, x, step.ws, accumulate=True)
 
     @staticmethod

@@ -350,12 +350,60 @@ def test_routing_and_experts():
         stack = lambda n: torch.tensor(np.stack([w[f"e{e}.{n}"] for e in range(E)]), dtype=torch.float32).cuda().to(dtype)
         hd = torch.tensor(h, dtype=torch.float32).cuda().to(dtype)
         y = torch.zeros((T, top, F), dtype=dtype, device="cuda")
-        K.experts_up(hd, stack("gate"), stack("up"), chosen, y)
+        w_gu = torch.cat([stack("gate"), stack("up")], dim=1).contiguous()
+        K.experts_up(hd, w_gu, chosen, y)
         x0 = rng.standard_normal((T, W)).astype(np.float32)
         x = torch.tensor(x0).cuda()
         K.experts_down(y, stack("down"), chosen, share, x)
         tol = 2e-5 if dtype == torch.float32 else 2e-2
         assert np.abs(x.cpu().numpy() - x0 - want).max() < tol * max(1.0, np.abs(want).max())
+
+
+def test_experts_in_their_order():
+    """The pairs of (token, slot) grouped by expert, their rows gathered, and the weighted outputs added back."""
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(8)
+    T, top, E, W = 130, 3, 7, 20
+    chosen = np.stack([rng.permutation(E)[:top] for _ in range(T)]).astype(np.int32)
+    chosen[chosen == 6] = chosen[0, 0]              # no token takes expert 6 (a token may take an expert twice here)
+    n = T * top
+    first = torch.zeros(E + 1, dtype=torch.int32, device="cuda")
+    order = torch.zeros(n, dtype=torch.int32, device="cuda")
+    place = torch.zeros(n, dtype=torch.int32, device="cuda")
+    K.experts_sort(dev_i(chosen), first, order, place, E)
+    f, o, p = first.cpu().numpy(), order.cpu().numpy(), place.cpu().numpy()
+    flat = chosen.reshape(-1)
+    assert f[0] == 0 and f[E] == n and np.array_equal(np.diff(f), np.bincount(flat, minlength=E))
+    assert sorted(o.tolist()) == list(range(n)) and np.array_equal(o[p], np.arange(n))
+    for e in range(E):
+        assert np.all(flat[o[f[e]:f[e + 1]]] == e)
+    h = rng.standard_normal((T, W)).astype(np.float32)
+    rows = torch.zeros((n, W), dtype=torch.float32, device="cuda")
+    K.experts_gather(dev_f(h), order, rows, top)
+    assert np.array_equal(rows.cpu().numpy(), h[o // top])
+    out = rng.standard_normal((n, W)).astype(np.float32)
+    share = rng.uniform(0, 1, (T, top)).astype(np.float32)
+    x0 = rng.standard_normal((T, W)).astype(np.float32)
+    x = dev_f(x0)
+    K.experts_combine(dev_f(out), place, dev_f(share), x)
+    want = x0 + (share[:, :, None].astype(np.float64) * out[p].reshape(T, top, W)).sum(axis=1)
+    assert np.abs(x.cpu().numpy() - want).max() < 1e-5
+
+
+def test_a_product_head_by_head():
+    from braidinfer_amd import kernels as K
+    rng = np.random.default_rng(9)
+    for T, H, N, K_, dtype, pad in ((70, 3, 40, 24, torch.bfloat16, 8), (5, 2, 130, 16, torch.bfloat16, 0), (33, 4, 10, 12, torch.bfloat16, 2),
+                                    (9, 5, 7, 13, torch.float32, 3), (1, 1, 96, 64, torch.bfloat16, 16)):
+        a = P.to_bf16(rng.standard_normal((T, H, K_ + pad)))
+        w = P.to_bf16(rng.standard_normal((H, N, K_)))
+        ad = torch.tensor(a, dtype=torch.float32).cuda().to(dtype)
+        od = torch.full((T, H, N + 5), 7.0, dtype=dtype, device="cuda")
+        K.head_linear(ad[:, :, :K_], torch.tensor(w, dtype=torch.float32).cuda().to(dtype), od[:, :, 2:2 + N])
+        want = np.einsum("thk,hnk->thn", a[:, :, :K_], w)
+        got = od.float().cpu().numpy()
+        assert np.abs(got[:, :, 2:2 + N] - want).max() < (1e-5 if dtype == torch.float32 else 0.01) * np.abs(want).max()
+        assert np.all(got[:, :, :2] == 7.0) and np.all(got[:, :, 2 + N:] == 7.0)          # nothing beside the view is touched
 
 
 def test_clamped_gated_unit():
