@@ -72,7 +72,9 @@ def measured_peaks(torch, K):
 LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_kv_write", "silu_mul", "residual_add", "gather_rows",
              "convert", "gemm", "gemm_swiglu", "gemm_norm_prepare", "gemm_norm_scaled", "attention_simple",
              "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16", "pwa_decode_bf16",
-             "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax"]
+             "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax", "wkv_scan", "wkv_scan_pieces", "shift_mix", "head_norm_gate", "tanh",
+             "latent_prepare", "head_linear", "route_topk", "experts_up", "experts_down", "experts_sort", "experts_gather",
+             "experts_combine", "experts_up_grouped", "experts_down_grouped", "clamped_glu", "add_bias_rows"]
 
 
 def kernel_share(torch, eng, entries_of, classes):
@@ -258,8 +260,11 @@ class Shape:
 # `--design kesitar`: prompt and single-token throughput of the Kesitar design at the sizes of a real model's
 # layers, beside Mistral (the library's closest model: grouped-query attention, gated feed-forward) with the same
 # width, heads, feed-forward and number of layers, and the time of every kernel launcher in one prompt and one
-# single-token step of each (run eagerly, bracketed by events).
+# single-token step of each (run eagerly, bracketed by events).  `--design sidirax`: the Sidirax design beside
+# Kesitar (the library's closest model: attention layers between linear recurrences, a sink in the softmax) at
+# equal width and layers; what is set beside a design is a Mistral configuration (a dict) or a preset's name.
 DESIGN_SIZES = {
+    "sidirax": {"1b": ("sidirax-1b", "kesitar-1b"), "7b": ("sidirax-7b", "kesitar-7b")},
     "kesitar": {
         "1b": ("kesitar-1b", dict(hidden_size=2048, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
                                   intermediate_size=5632, vocab_size=32768, rope_theta=10000.0, rms_norm_eps=1e-6,
@@ -388,7 +393,8 @@ def design_comparison(args) -> int:
     import torch
     import braidinfer_amd as B
     sizes = DESIGN_SIZES[args.design]
-    line = {"metric": f"{args.design} beside mistral at equal size: prefill and decode tokens/s, bf16, random weights",
+    beside = "kesitar" if args.design == "sidirax" else "mistral"
+    line = {"metric": f"{args.design} beside {beside} at equal size: prefill and decode tokens/s, bf16, random weights",
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "layers": args.layers or 8,
             "steps": args.steps, "warmup": args.warmup, "sizes": {}}
     prompts = [2048, 8192]
@@ -397,12 +403,18 @@ def design_comparison(args) -> int:
         L = args.layers or 8
         full = B.any_preset(preset_name)
         cfg = B.any_preset(preset_name, layers=[dict(l) for l in full.layers[:L]])
-        mistral = B.MistralConfig.from_dict(dict(like, num_hidden_layers=L))
         got = {}
         got[args.design] = measure_design(torch, B, f"{preset_name} ({L} layers)", cfg, cfg.vocab, prompts, [8, 64], 1024,
                                           args.steps, args.warmup)
-        got["mistral"] = measure_design(torch, B, f"mistral of that size ({L} layers)", mistral, mistral.vocab_size, prompts,
-                                        [8, 64], 1024, args.steps, args.warmup)
+        if isinstance(like, str):            # another design's preset of that size
+            whole = B.any_preset(like)
+            other = B.any_preset(like, layers=[dict(l) for l in whole.layers[:L]])
+            got[like.split("-")[0]] = measure_design(torch, B, f"{like} ({L} layers)", other, other.vocab, prompts, [8, 64], 1024,
+                                                     args.steps, args.warmup)
+        else:
+            mistral = B.MistralConfig.from_dict(dict(like, num_hidden_layers=L))
+            got["mistral"] = measure_design(torch, B, f"mistral of that size ({L} layers)", mistral, mistral.vocab_size, prompts,
+                                            [8, 64], 1024, args.steps, args.warmup)
         line["sizes"][size] = got
     print(json.dumps(line), flush=True)
     return 0

@@ -331,11 +331,15 @@ extern "C" int br_glr_head_norm(const float* o, const float* w, void* y, int y_i
 // one value, 4 RPL multiply-adds and the four moves that add the row groups' shares of o_t[c].
 //
 // rows [T, width] hold r | k | v | z at the column offsets 0, H d, 2 H d, 2 H d + H e (floats).
-template <int RPL, int TC, bool V4>
+//
+// LOCAL (the first pass over a long prompt cut into pieces, see `br_wkv_scan_pieces`): the state starts at zero,
+// nothing is written to o, and beside the piece's last state the products of its decays go to `decay`
+// ([sequences of the launch][head][16 RPL], in row order).
+template <int RPL, int TC, bool V4, bool LOCAL>
 __global__ __launch_bounds__(256) void wkv_scan_kernel(
     const float* __restrict__ rows, const float* __restrict__ w0, const float* __restrict__ bonus,
     float* __restrict__ o, float* __restrict__ state, const int* __restrict__ cu_seqlens,
-    const int* __restrict__ slots, int H, int d, int e, int width, size_t slot_stride) {
+    const int* __restrict__ slots, int H, int d, int e, int width, size_t slot_stride, float* __restrict__ decay) {
     constexpr int DP = RPL * 16;
     constexpr int NL = TC * DP / 1024;
     extern __shared__ float lds[];
@@ -351,7 +355,7 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(
     const int t0 = cu_seqlens[s], t1 = cu_seqlens[s + 1];
     const bool live = c < e;
     if (slot < 0) {                                // padding: no state behind it; its rows of o are zero
-        if (g == 0 && live) for (int t = t0; t < t1; ++t) o[(size_t)t * H * e + h * e + c] = 0.f;
+        if (!LOCAL && g == 0 && live) for (int t = t0; t < t1; ++t) o[(size_t)t * H * e + h * e + c] = 0.f;
         return;
     }
     const int ncb4 = (e + 3) >> 2;
@@ -359,10 +363,13 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(
     float st[RPL], ub[RPL];
 #pragma unroll
     for (int k = 0; k < RPL; ++k) {
-        st[k] = cb4 < ncb4 ? S[(size_t)k * 64] : 0.f;
+        st[k] = (!LOCAL && cb4 < ncb4) ? S[(size_t)k * 64] : 0.f;
         const int r = g * RPL + k;
         ub[k] = r < d ? bonus[h * d + r] : 0.f;
     }
+    float dec[LOCAL ? RPL : 1];
+#pragma unroll
+    for (int k = 0; k < (LOCAL ? RPL : 1); ++k) dec[k] = 1.f;
     const int hd = H * d, he = H * e;
     int l_tt[NL], l_r4[NL];
     float b4[NL][4];
@@ -444,17 +451,21 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(
             for (int k4 = 0; k4 < RPL / 4; ++k4) {
                 const f32x4 wv = *(const f32x4*)(wp + (size_t)tt * DP + 4 * k4);
                 const f32x4 kv4 = *(const f32x4*)(kp + (size_t)tt * DP + 4 * k4);
-                const f32x4 rv4 = *(const f32x4*)(rp + (size_t)tt * DP + 4 * k4);
+                f32x4 rv4 = {0.f, 0.f, 0.f, 0.f};
+                if (!LOCAL) rv4 = *(const f32x4*)(rp + (size_t)tt * DP + 4 * k4);
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
                     const float kv = kv4[x] * vc;
-                    sum = fmaf(rv4[x], fmaf(ub[4 * k4 + x], kv, st[4 * k4 + x]), sum);
+                    if (LOCAL) dec[LOCAL ? 4 * k4 + x : 0] *= wv[x];
+                    else sum = fmaf(rv4[x], fmaf(ub[4 * k4 + x], kv, st[4 * k4 + x]), sum);
                     st[4 * k4 + x] = fmaf(wv[x], st[4 * k4 + x], kv);
                 }
             }
-            sum = glr_row16_sum(sum);
-            if (g == 0 && live) orow[0] = sum;
-            orow += he;
+            if (!LOCAL) {
+                sum = glr_row16_sum(sum);
+                if (g == 0 && live) orow[0] = sum;
+                orow += he;
+            }
         }
         if (more) stage(buf ^ 1);
         __syncthreads();
@@ -464,24 +475,29 @@ __global__ __launch_bounds__(256) void wkv_scan_kernel(
 #pragma unroll
         for (int k = 0; k < RPL; ++k) S[(size_t)k * 64] = st[k];
     }
+    if (LOCAL && cb16 == 0 && wave == 0 && cg == 0) {
+        float* dr = decay + ((size_t)s * H + h) * DP + g * RPL;
+#pragma unroll
+        for (int k = 0; k < (LOCAL ? RPL : 1); ++k) dr[k] = dec[k];
+    }
 }
 
 // rows [T, width] float: r | k | v | z at 0, H d, 2 H d, 2 H d + H e; w0 and bonus float [H d]; o float [T, H e];
 // `slot_stride`: floats from one slot's state to the next (at least H * ceil(e / 4) * rows per lane * 64).
-extern "C" int br_wkv_scan(const float* rows, const float* w0, const float* bonus, float* o, float* state,
+template <bool LOCAL>
+static int wkv_scan_launch(const float* rows, const float* w0, const float* bonus, float* o, float* state,
                            const int* cu_seqlens, const int* slots, int B, int H, int d, int e, int width,
-                           size_t slot_stride, hipStream_t s) {
-    if (B <= 0) return BR_OK;
+                           size_t slot_stride, float* decay, hipStream_t s) {
     const int ncb4 = (e + 3) / 4, rpl = glr_rpl(d);
     if (H <= 0 || H > 65535 || d <= 0 || e <= 0 || d > 512 || (e + 15) / 16 > 65535 || width < 3 * H * d + H * e ||
-        slot_stride < (size_t)H * ncb4 * rpl * 64 || !w0 || !bonus)
+        slot_stride < (size_t)H * ncb4 * rpl * 64 || !w0 || !bonus || (LOCAL && !decay))
         return BR_BAD_ARG;
     dim3 grid(B, H, (e + 15) / 16);
     const bool v4 = d % 4 == 0 && e % 4 == 0 && width % 4 == 0 && ((uintptr_t)rows % 16) == 0;
 #define WKV_SCAN(R, TC) do { \
         const size_t lds = (size_t)(6 * TC * R * 16 + 2 * TC * 16) * sizeof(float); \
-        if (v4) wkv_scan_kernel<R, TC, true><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride); \
-        else wkv_scan_kernel<R, TC, false><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride); \
+        if (v4) wkv_scan_kernel<R, TC, true, LOCAL><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride, decay); \
+        else wkv_scan_kernel<R, TC, false, LOCAL><<<grid, 256, lds, s>>>(rows, w0, bonus, o, state, cu_seqlens, slots, H, d, e, width, slot_stride, decay); \
     } while (0)
     if (rpl == 4) WKV_SCAN(4, 16);
     else if (rpl == 8) WKV_SCAN(8, 16);
@@ -489,6 +505,36 @@ extern "C" int br_wkv_scan(const float* rows, const float* w0, const float* bonu
     else WKV_SCAN(32, 4);
 #undef WKV_SCAN
     return br_check_launch();
+}
+
+extern "C" int br_wkv_scan(const float* rows, const float* w0, const float* bonus, float* o, float* state,
+                           const int* cu_seqlens, const int* slots, int B, int H, int d, int e, int width,
+                           size_t slot_stride, hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    return wkv_scan_launch<false>(rows, w0, bonus, o, state, cu_seqlens, slots, B, H, d, e, width, slot_stride, nullptr, s);
+}
+
+// A step of long prompts with every sequence cut into `pieces` pieces that run side by side, as `br_glr_scan_pieces`
+// does for its recurrence: a walk from zero (last state L, decay products D), s_(c+1) = D_c s_c + L_c by
+// `glr_carry_kernel` (the bonus touches o only, never the state), a second walk from the true states that writes o.
+extern "C" int br_wkv_scan_pieces(const float* rows, const float* w0, const float* bonus, float* o, float* state,
+                                  const int* slots, const int* piece_cu, const int* piece_slots, float* piece_state,
+                                  float* decay, int B, int pieces, int H, int d, int e, int width, size_t slot_stride,
+                                  hipStream_t s) {
+    if (B <= 0) return BR_OK;
+    if (pieces <= 0 || (long long)B * pieces > 65535) return BR_BAD_ARG;
+    const int ncb4 = (e + 3) / 4, rpl = glr_rpl(d);
+    const size_t piece_stride = (size_t)H * ncb4 * rpl * 64;
+    int rc = wkv_scan_launch<true>(rows, w0, bonus, o, piece_state, piece_cu, piece_slots, B * pieces, H, d, e, width,
+                                   piece_stride, decay, s);
+    if (rc != BR_OK) return rc;
+    if ((long long)H * ncb4 > 65535 || slot_stride < piece_stride) return BR_BAD_ARG;
+    glr_carry_kernel<<<dim3(B, H * ncb4), 64, 0, s>>>(state, slot_stride, slots, piece_state, piece_stride, decay, pieces, H,
+                                                      ncb4, rpl);
+    rc = br_check_launch();
+    if (rc != BR_OK) return rc;
+    return wkv_scan_launch<false>(rows, w0, bonus, o, piece_state, piece_cu, piece_slots, B * pieces, H, d, e, width,
+                                  piece_stride, nullptr, s);
 }
 
 // ------------------------------------------------------------- shifted mixes --------

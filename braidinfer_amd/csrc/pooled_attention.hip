@@ -734,7 +734,17 @@ template <int NBK>
 static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStream_t s, const bf16* q, bf16* out, const int* slots,
                                const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
                                int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds) {
-#define PWA_GO(V) pwa_decode_kernel<NBK, V><<<grid, 64 * PWA_DW, head_lds + lds_of_nbv16 * V, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks)
+    // merges beyond 64 KB of LDS (many query heads to a kv head with wide values) are asked for once per kernel
+#define PWA_GO(V) do { \
+        auto kern = pwa_decode_kernel<NBK, V>; \
+        const size_t lds = head_lds + lds_of_nbv16 * V; \
+        static size_t have = 65536; \
+        if (lds > have) { \
+            if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
+            have = lds; \
+        } \
+        kern<<<grid, 64 * PWA_DW, lds, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks); \
+    } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
     else if (nbv <= 3) PWA_GO(3);
@@ -744,14 +754,15 @@ static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStrea
     return br_check_launch();
 }
 
-// Bytes of LDS the merge of `pwa_decode_kernel` needs for these sizes (the launcher refuses more than 64 KB).
+// Bytes of LDS the merge of `pwa_decode_kernel` needs for these sizes (the launcher refuses more than 144 KB of a
+// compute unit's 160).
 static size_t pwa_decode_lds(int G, int dv) {
     const int nbv = (dv + 31) / 32, v = nbv <= 4 ? nbv : 8;
     return (size_t)(2 * PWA_DW * 2 * G + PWA_DW * v * 16 * 2 * G) * sizeof(float);
 }
 extern "C" int br_pwa_decode_takes(int nq, int nkv, int dk, int dv) {
     if (nq <= 0 || nkv <= 0 || nq % nkv || nq / nkv > 32 || dk <= 0 || dv <= 0 || dk > 256 || dv > 256 || dk % 8 || dv % 4) return 0;
-    return pwa_decode_lds(nq / nkv, dv) <= 65536;
+    return pwa_decode_lds(nq / nkv, dv) <= 147456;
 }
 
 extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, const int* ctx_lens, const int* block_table,

@@ -224,3 +224,123 @@ extern "C" int br_experts_combine(const float* out, const int* place, const floa
     experts_combine_kernel<<<dim3(T, (W + 255) / 256), 256, 0, s>>>(out, place, share, x, W, top);
     return br_check_launch();
 }
+
+// ------------------------------------------- few tokens, every expert read once -----
+// bfloat16 on the matrix cores, for steps whose pairs were grouped by `sort` on the device (nothing comes back to
+// the host, so the step can be recorded): a workgroup owns 32 output rows of one expert's matrix and walks that
+// expert's pairs 32 at a time, so an expert's weights are read once per 32 of its pairs instead of once per pair.
+// Its four waves share k (wave w takes the k-steps of 16 numbered w, w + 4, ...), v_mfma_f32_32x32x16_bf16 with
+// the weight rows as the first operand, both operands straight from memory; the waves' sums meet in LDS in wave
+// order.  Experts without pairs cost a workgroup a load and a compare.
+//
+// `up`: rows of h gathered through `order` (pair -> token = pair / top), gate and up rows of the same f in the same
+// lane, y[p, f] = silu(g) * u in the experts' order.  grid (E, ceil(F / 32)).
+__global__ __launch_bounds__(256) void experts_up_grouped_kernel(const bf16* __restrict__ h, const bf16* __restrict__ w_gu,
+                                                                 const int* __restrict__ first, const int* __restrict__ order,
+                                                                 bf16* __restrict__ y, int W, int F, int top) {
+    __shared__ float red[3][2][16][64];
+    const int e = blockIdx.x, f0 = blockIdx.y * 32;
+    const int p0 = first[e], p1 = first[e + 1];
+    if (p0 >= p1) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, g = lane >> 5;
+    const int f = f0 + c;
+    const bf16* wg = w_gu + ((size_t)e * 2 * F + (f < F ? f : F - 1)) * W;
+    const bf16* wu = wg + (size_t)F * W;
+    bf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+    for (int pb = p0; pb < p1; pb += 32) {
+        const int p = pb + c;
+        const bf16* arow = h + (size_t)(order[p < p1 ? p : p1 - 1] / top) * W;
+        f32x16 ag, au;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { ag[r] = 0.f; au[r] = 0.f; }
+        for (int k0 = wave * 16; k0 < W; k0 += 64) {
+            const int k = k0 + 8 * g;
+            const bool on = k < W;
+            const bf16x8 af = (on && p < p1) ? *(const bf16x8*)(arow + k) : zero;
+            const bf16x8 gf = (on && f < F) ? *(const bf16x8*)(wg + k) : zero;
+            const bf16x8 uf = (on && f < F) ? *(const bf16x8*)(wu + k) : zero;
+            ag = __builtin_amdgcn_mfma_f32_32x32x16_bf16(gf, af, ag, 0, 0, 0);
+            au = __builtin_amdgcn_mfma_f32_32x32x16_bf16(uf, af, au, 0, 0, 0);
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { red[wave - 1][0][r][lane] = ag[r]; red[wave - 1][1][r][lane] = au[r]; }
+        }
+        __syncthreads();
+        if (wave == 0 && p < p1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float gs = ((ag[r] + red[0][0][r][lane]) + red[1][0][r][lane]) + red[2][0][r][lane];
+                const float us = ((au[r] + red[0][1][r][lane]) + red[1][1][r][lane]) + red[2][1][r][lane];
+                const int ff = f0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (ff < F) y[(size_t)p * F + ff] = (bf16)(gs / (1.0f + expf(-gs)) * us);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// `down`: out[p, n] = W_d[e] y[p, :] as float for the pairs in the experts' order (`combine` adds them to the rows).
+// grid (E, ceil(W / 32)).
+__global__ __launch_bounds__(256) void experts_down_grouped_kernel(const bf16* __restrict__ y, const bf16* __restrict__ w_down,
+                                                                   const int* __restrict__ first, float* __restrict__ out,
+                                                                   int W, int F) {
+    __shared__ float red[3][16][64];
+    const int e = blockIdx.x, n0 = blockIdx.y * 32;
+    const int p0 = first[e], p1 = first[e + 1];
+    if (p0 >= p1) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, g = lane >> 5;
+    const int n = n0 + c;
+    const bf16* wr = w_down + ((size_t)e * W + (n < W ? n : W - 1)) * F;
+    bf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+    for (int pb = p0; pb < p1; pb += 32) {
+        const int p = pb + c;
+        const bf16* arow = y + (size_t)(p < p1 ? p : p1 - 1) * F;
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        for (int k0 = wave * 16; k0 < F; k0 += 64) {
+            const int k = k0 + 8 * g;
+            const bool on = k < F;
+            const bf16x8 af = (on && p < p1) ? *(const bf16x8*)(arow + k) : zero;
+            const bf16x8 wf = (on && n < W) ? *(const bf16x8*)(wr + k) : zero;
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, af, acc, 0, 0, 0);
+        }
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) red[wave - 1][r][lane] = acc[r];
+        }
+        __syncthreads();
+        if (wave == 0 && p < p1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int nn = n0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (nn < W) out[(size_t)p * W + nn] = ((acc[r] + red[0][r][lane]) + red[1][r][lane]) + red[2][r][lane];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Whether the grouped kernels take these sizes: rows of 16 bytes' multiples.
+extern "C" int br_experts_grouped_takes(int W, int F) { return W > 0 && F > 0 && W % 8 == 0 && F % 8 == 0; }
+
+extern "C" int br_experts_up_grouped(const void* h, const void* w_gu, const int* first, const int* order, void* y, int E,
+                                     int W, int F, int top, hipStream_t s) {
+    if (!br_experts_grouped_takes(W, F) || E <= 0 || top <= 0 || (F + 31) / 32 > 65535) return BR_BAD_ARG;
+    experts_up_grouped_kernel<<<dim3(E, (F + 31) / 32), 256, 0, s>>>((const bf16*)h, (const bf16*)w_gu, first, order, (bf16*)y, W, F, top);
+    return br_check_launch();
+}
+
+extern "C" int br_experts_down_grouped(const void* y, const void* w_down, const int* first, float* out, int E, int W, int F,
+                                       hipStream_t s) {
+    if (!br_experts_grouped_takes(W, F) || E <= 0 || (W + 31) / 32 > 65535) return BR_BAD_ARG;
+    experts_down_grouped_kernel<<<dim3(E, (W + 31) / 32), 256, 0, s>>>((const bf16*)y, (const bf16*)w_down, first, out, W, F);
+    return br_check_launch();
+}

@@ -765,6 +765,31 @@ def wkv_scan(rows: torch.Tensor, w0: torch.Tensor, bonus: torch.Tensor, out: tor
              rows.shape[1], state.stride(0), _stream()), "wkv_scan")
 
 
+def wkv_scan_pieces(rows: torch.Tensor, w0: torch.Tensor, bonus: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+                    slots: torch.Tensor, piece_cu: torch.Tensor, piece_slots: torch.Tensor, piece_state: torch.Tensor,
+                    decay: torch.Tensor, B: int, pieces: int, H: int, d: int, e: int) -> None:
+    """`wkv_scan` of a step of long prompts with every sequence cut into `pieces` pieces that are walked side by side
+    (twice: from a zero state, then from their true first states); arrays as for `glr_scan_pieces`."""
+    _dev("wkv_scan_pieces", rows, w0, bonus, out, slots, piece_cu, piece_slots, piece_state, decay)
+    T = rows.shape[0]
+    shape = glr_state_shape(H, d, e)
+    need = 1
+    for n in shape:
+        need *= n
+    _req(state.is_cuda and state.dim() == 2 and state.shape[1] >= need and state.stride(1) == 1, "wkv_scan_pieces: state [slots, >= the head states' floats]")
+    _req(rows.dtype == out.dtype == state.dtype == piece_state.dtype == decay.dtype == torch.float32, "wkv_scan_pieces: float32 only")
+    _req(rows.dim() == 2 and rows.shape[1] >= 3 * H * d + H * e and out.shape == (T, H * e), "wkv_scan_pieces: rows [T, >= 3*H*d + H*e], out [T, H*e]")
+    _req(piece_state.shape == (B * pieces,) + tuple(shape) and decay.shape == (B * pieces, H, 16 * glr_rows_per_lane(d)),
+         "wkv_scan_pieces: scratch of the wrong size")
+    _req(piece_cu.dtype == piece_slots.dtype == torch.int32 and piece_cu.numel() == B * pieces + 1 and piece_slots.numel() == B * pieces
+         and slots.numel() >= B, "wkv_scan_pieces: piece arrays int32 [B*pieces + 1] and [B*pieces]")
+    for v in (w0, bonus):
+        _req(v.dtype == torch.float32 and v.numel() == H * d, "wkv_scan_pieces: w0 and bonus float32 [H*d]")
+    f = _fn("gated_recurrence", "br_wkv_scan_pieces", [_P] * 10 + [c_int] * 6 + [c_size_t, _P])
+    _check(f(_ptr(rows), _ptr(w0), _ptr(bonus), _ptr(out), _ptr(state), _ptr(slots), _ptr(piece_cu), _ptr(piece_slots),
+             _ptr(piece_state), _ptr(decay), B, pieces, H, d, e, rows.shape[1], state.stride(0), _stream()), "wkv_scan_pieces")
+
+
 def shift_mix(h: torch.Tensor, mu: torch.Tensor, out: torch.Tensor, kept: torch.Tensor, seq_of_token: torch.Tensor,
               cu_seqlens: torch.Tensor, slots: torch.Tensor, B: int, single_tokens: bool) -> None:
     """out[s, t] = h[t] + (h'[t] - h[t]) * mu[s], h' the row of the token before in its sequence, and before a step's
@@ -916,6 +941,36 @@ def experts_down(y: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, sh
     _req(top * F <= 16384, "experts_down: more than 16,384 inner elements a token")
     f = _fn("routed_experts", "br_experts_down", [_P, _P, _P, _P, _P] + [c_int] * 5 + [_P])
     _check(f(_ptr(y), _ptr(w_down), _ptr(chosen), _ptr(share), _ptr(x), _is_bf16(y, "experts_down"), T, W, F, top, _stream()), "experts_down")
+
+
+def experts_grouped_takes(dtype: torch.dtype, W: int, F: int) -> bool:
+    """Whether the kernels that read every expert once take these sizes (bfloat16, widths in steps of 8)."""
+    return dtype == torch.bfloat16 and W % 8 == 0 and F % 8 == 0
+
+
+def experts_up_grouped(h: torch.Tensor, w_gu: torch.Tensor, first: torch.Tensor, order: torch.Tensor, y: torch.Tensor, top: int) -> None:
+    """y[p] = silu(W_gate[e] h[t]) * (W_up[e] h[t]) for the pairs p of `experts_sort` (t = order[p] // top, e the
+    expert whose run holds p); y [pairs, F] in the experts' order."""
+    _dev("experts_up_grouped", h, w_gu, first, order, y)
+    T, W = h.shape
+    E, F2, _ = w_gu.shape
+    n = order.numel()
+    _req(experts_grouped_takes(h.dtype, W, F2 // 2) and w_gu.dtype == y.dtype == torch.bfloat16, "experts_up_grouped: bfloat16, widths in steps of 8")
+    _req(w_gu.shape == (E, F2, W) and y.shape == (n, F2 // 2) and first.numel() == E + 1 and n == T * top
+         and first.dtype == order.dtype == torch.int32, "experts_up_grouped: shapes")
+    f = _fn("routed_experts", "br_experts_up_grouped", [_P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P])
+    _check(f(_ptr(h), _ptr(w_gu), _ptr(first), _ptr(order), _ptr(y), E, W, F2 // 2, top, _stream()), "experts_up_grouped")
+
+
+def experts_down_grouped(y: torch.Tensor, w_down: torch.Tensor, first: torch.Tensor, out: torch.Tensor) -> None:
+    """out[p] = W_down[e] y[p] (float) for the pairs in the experts' order."""
+    _dev("experts_down_grouped", y, w_down, first, out)
+    n, F = y.shape
+    E, W, _ = w_down.shape
+    _req(experts_grouped_takes(y.dtype, W, F) and w_down.dtype == torch.bfloat16 and out.dtype == torch.float32, "experts_down_grouped: types")
+    _req(w_down.shape == (E, W, F) and out.shape == (n, W) and first.numel() == E + 1 and first.dtype == torch.int32, "experts_down_grouped: shapes")
+    f = _fn("routed_experts", "br_experts_down_grouped", [_P, _P, _P, _P, c_int, c_int, c_int, _P])
+    _check(f(_ptr(y), _ptr(w_down), _ptr(first), _ptr(out), E, W, F, _stream()), "experts_down_grouped")
 
 
 # ------------------------------------------------------------- clamped gated unit -----

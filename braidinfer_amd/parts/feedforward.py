@@ -11,6 +11,7 @@ Routed experts: router scores z = W_r n + b_r in float; a token takes the `top` 
 with an expert W_d (silu(W_g n) * (W_u n)) without biases.  The reference has neither."""
 from __future__ import annotations
 
+import os
 from typing import Dict, List, Optional
 
 import torch
@@ -166,29 +167,42 @@ class RoutedExperts(FeedForward):
         chosen = step.ws.get("moe_chosen", (T, self.top), torch.int32)
         share = step.ws.get("moe_share", (T, self.top), torch.float32)
         K.route_topk(scores, self.b_router, chosen, share, self.top)
-        if step.is_decode or T < self.BY_EXPERT_FROM:
+        few = step.is_decode or T < int(os.environ.get("BRAIDINFER_BY_EXPERT_FROM", str(self.BY_EXPERT_FROM)))
+        if few and not K.experts_grouped_takes(dt, self.H, self.I):
+            # every pair reads its expert's rows itself: the 32-bit path, and widths the grouped kernels do not take
             y = step.ws.get("moe_y", (T, self.top, self.I), dt)
             K.experts_up(h, self.w_gu, chosen, y)
             K.experts_down(y, self.w_down, chosen, share, x)
             return
-        # expert by expert: the pairs sorted by expert on the device, the experts' row counts read by the host
+        # the pairs sorted by expert on the device
         n = T * self.top
         first = step.ws.get("moe_first", (self.E + 1,), torch.int32)
         order = step.ws.get("moe_order", (n,), torch.int32)
         place = step.ws.get("moe_place", (n,), torch.int32)
         K.experts_sort(chosen, first, order, place, self.E)
+        if few:
+            # few tokens: an expert's weights are read once for all its pairs, nothing goes back to the host
+            y = step.ws.get("moe_y", (n, self.I), dt)
+            K.experts_up_grouped(h, self.w_gu, first, order, y, self.top)
+            out = step.ws.get("moe_out", (n, self.H), torch.float32)
+            K.experts_down_grouped(y, self.w_down, first, out)
+            K.experts_combine(out, place, share, x)
+            return
+        # many tokens: expert by expert through the matrix products, the experts' row counts read by the host
         rows = step.ws.get("moe_rows", (n, self.H), dt)
         K.experts_gather(h, order, rows, self.top)
         starts = first.tolist()
         gu = step.ws.get("moe_gu", (n, 2 * self.I), dt)
         act = step.ws.get("moe_act", (n, self.I), dt)
         out = step.ws.get("moe_out", (n, self.H), torch.float32)
+        scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if dt == torch.bfloat16 else None
         for e in range(self.E):
             a, b = starts[e], starts[e + 1]
             if b > a:
-                linear(rows[a:b], self.w_gu[e], gu[a:b], step.ws)
+                sc = scratch if 16 < b - a <= 1024 else None          # products that may be cut along k
+                K.gemm(rows[a:b], self.w_gu[e], gu[a:b], scratch=sc)
                 K.silu_mul(gu[a:b], act[a:b])
-                linear(act[a:b], self.w_down[e], out[a:b], step.ws)
+                K.gemm(act[a:b], self.w_down[e], out[a:b], scratch=sc)
         K.experts_combine(out, place, share, x)
 
 

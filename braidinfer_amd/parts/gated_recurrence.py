@@ -29,6 +29,21 @@ from .base import Mixer, MixerContext, Runtime, register_part
 from .linear import fused_layout, linear, stream_layout
 
 
+def pieces_for(step, units_per_sequence: int, min_piece: int) -> int:
+    """Into how many pieces a step's sequences are cut so that a recurrence's walk fills the chip: a workgroup walks 16
+    columns of a head's state for one sequence (`units_per_sequence` of them a sequence), and a lone prompt of a small
+    model has a few dozen.  One piece (the plain walk) for single tokens, short steps and batches that fill the chip."""
+    if step.is_decode or step.max_new < 4 * min_piece:
+        return 1
+    # a workgroup is four waves, one to a SIMD, and a lone wave waits out every latency of its token loop, so
+    # pieces are asked for until four workgroups share a compute unit (BRAIDINFER_GLR_FILL, for measurements;
+    # a prompt of 8,192 tokens through 8 HGRN2 layers of width 2,048 / 4,096: 17.8 / 43.3 ms at 1, 13.7 / 40.2 at 2,
+    # 12.9 / 38.4 at 4, 12.8 / 38.1 at 8)
+    units = step.n_seqs * units_per_sequence
+    want = (int(os.environ.get("BRAIDINFER_GLR_FILL", "4")) * K.device_cus()) // max(1, units)
+    return max(1, min(want, step.max_new // min_piece, 16, 65535 // max(1, step.n_seqs)))
+
+
 class HGRN2(Mixer):
     graph_safe = True
     through_linear_only = True
@@ -71,18 +86,7 @@ class HGRN2(Mixer):
     MIN_PIECE = 128          # tokens: shorter pieces do not pay for the second walk
 
     def pieces_for(self, step) -> int:
-        """Into how many pieces a step's sequences are cut so that the walk fills the chip: a workgroup walks 16
-        columns of a head's state for one sequence, and a lone prompt of a small model has a few dozen of them.
-        One piece (the plain walk) for single tokens, short steps and batches that fill the chip already."""
-        if step.is_decode or step.max_new < 4 * self.MIN_PIECE:
-            return 1
-        # a workgroup is four waves, one to a SIMD, and a lone wave waits out every latency of its token loop, so
-        # pieces are asked for until four workgroups share a compute unit (BRAIDINFER_GLR_FILL, for measurements;
-        # a prompt of 8,192 tokens through 8 layers of width 2,048 / 4,096: 17.8 / 43.3 ms at 1, 13.7 / 40.2 at 2,
-        # 12.9 / 38.4 at 4, 12.8 / 38.1 at 8)
-        units = step.n_seqs * self.nh * -(-self.e // 16)
-        want = (int(os.environ.get("BRAIDINFER_GLR_FILL", "4")) * K.device_cus()) // max(1, units)
-        return max(1, min(want, step.max_new // self.MIN_PIECE, 16, 65535 // max(1, step.n_seqs)))
+        return pieces_for(step, self.nh * -(-self.e // 16), self.MIN_PIECE)
 
     @staticmethod
     def _piece_arrays(step, pieces: int):

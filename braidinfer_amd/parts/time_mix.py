@@ -27,6 +27,7 @@ from ..cache import StateNeed
 from ..errors import ConfigError, StepError
 from ..weights import TensorSpec
 from .base import Mixer, MixerContext, Runtime, register_part
+from .gated_recurrence import HGRN2, pieces_for
 from .linear import linear, stream_layout
 
 BRANCHES = ("r", "k", "v", "g", "w")
@@ -76,6 +77,8 @@ class WKVTimeMix(Mixer):
         self.u = rt.own(tensors[prefix + n["u"]].to(torch.float32).reshape(-1))
         self.norm_w = rt.own(tensors[prefix + n["norm"]].to(torch.float32).reshape(-1))
 
+    MIN_PIECE = 128          # tokens: shorter pieces do not pay for the second walk
+
     def state_need(self) -> StateNeed:
         # the heads' states as the scan keeps them, then the last token's input
         return StateNeed((self.state_floats + self.H,), torch.float32)
@@ -99,7 +102,17 @@ class WKVTimeMix(Mixer):
         K.tanh(low, low_t)
         linear(low_t, self.w["w2"], rows[:, 3 * hd:4 * hd], step.ws)
         o = step.ws.get("wkv_o", (T, hd), torch.float32)
-        K.wkv_scan(rows, self.w0, self.u, o, state, step.cu_seqlens, step.slots, step.n_seqs, self.nh, self.d, self.d)
+        pieces = pieces_for(step, self.nh * -(-self.d // 16), self.MIN_PIECE)
+        if pieces > 1:
+            # long prompts: every sequence cut into pieces that are walked side by side, twice
+            cu, numbers = HGRN2._piece_arrays(step, pieces)
+            n = step.n_seqs * pieces
+            piece_state = step.ws.get("wkv_piece_state", (n,) + tuple(K.glr_state_shape(self.nh, self.d, self.d)), torch.float32)
+            decay = step.ws.get("wkv_decay", (n, self.nh, 16 * K.glr_rows_per_lane(self.d)), torch.float32)
+            K.wkv_scan_pieces(rows, self.w0, self.u, o, state, step.slots, cu, numbers, piece_state, decay, step.n_seqs, pieces,
+                              self.nh, self.d, self.d)
+        else:
+            K.wkv_scan(rows, self.w0, self.u, o, state, step.cu_seqlens, step.slots, step.n_seqs, self.nh, self.d, self.d)
         y = step.ws.get("wkv_y", (T, hd), dt)
         K.head_norm_gate(o, self.norm_w, rows[:, 4 * hd:5 * hd], y, self.nh, self.d, self.eps)
         linear(y, self.w_o, x, step.ws, accumulate=True)

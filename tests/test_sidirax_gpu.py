@@ -329,7 +329,7 @@ def test_routing_and_experts():
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(5)
     for T, W, F, E, top, dtype in ((9, 50, 20, 7, 3, torch.float32), (4, 64, 24, 70, 5, torch.float32), (3, 32, 16, 2, 2, torch.float32),
-                                   (6, 64, 32, 8, 1, torch.bfloat16)):
+                                   (6, 64, 32, 8, 1, torch.bfloat16), (70, 72, 40, 5, 3, torch.bfloat16)):
         h = P.to_bf16(rng.standard_normal((T, W)))
         w = {"router": P.to_bf16(rng.standard_normal((E, W))), "router.b": P.to_bf16(rng.standard_normal(E))}
         w["router"][1] = w["router"][0]                       # two experts that always tie: the lower number goes first
@@ -357,6 +357,19 @@ def test_routing_and_experts():
         K.experts_down(y, stack("down"), chosen, share, x)
         tol = 2e-5 if dtype == torch.float32 else 2e-2
         assert np.abs(x.cpu().numpy() - x0 - want).max() < tol * max(1.0, np.abs(want).max())
+        if K.experts_grouped_takes(dtype, W, F):
+            # the same through the kernels that read every expert once
+            n = T * top
+            first, order, place = (torch.zeros(k, dtype=torch.int32, device="cuda") for k in (E + 1, n, n))
+            K.experts_sort(chosen, first, order, place, E)
+            y2 = torch.zeros((n, F), dtype=dtype, device="cuda")
+            K.experts_up_grouped(hd, w_gu, first, order, y2, top)
+            assert np.abs(y2[place.long()].float().cpu().numpy().reshape(T, top, F) - y.float().cpu().numpy()).max() < 0.02 * float(y.float().abs().max())
+            out = torch.zeros((n, W), dtype=torch.float32, device="cuda")
+            K.experts_down_grouped(y2, stack("down"), first, out)
+            x2 = torch.tensor(x0).cuda()
+            K.experts_combine(out, place, share, x2)
+            assert np.abs(x2.cpu().numpy() - x0 - want).max() < tol * max(1.0, np.abs(want).max())
 
 
 def test_experts_in_their_order():
@@ -490,7 +503,8 @@ def plain_latent(q, dkv, cw, sinks, H, D, DR, R, freqs, mag, scale, absorb):
     return P.sink_softmax_attention(qq, k, v, scale, sinks)
 
 
-@pytest.mark.parametrize("H,D,DR,R,rot", [(4, 16, 8, 24, 8), (1, 10, 6, 14, 6), (3, 12, 4, 10, 2), (2, 8, 16, 40, 16), (2, 5, 0, 8, 0)])
+@pytest.mark.parametrize("H,D,DR,R,rot", [(4, 16, 8, 24, 8), (1, 10, 6, 14, 6), (3, 12, 4, 10, 2), (2, 8, 16, 40, 16), (2, 5, 0, 8, 0),
+                                          (16, 8, 32, 160, 32)])
 def test_latent_attention_kernels(H, D, DR, R, rot):
     """prepare (norm, rotation, cache rows) and the attention kernels with a learnt sink a head, against the plain
     attention with expanded keys: whole, in portions across page borders, and token by token."""
