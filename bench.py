@@ -74,7 +74,7 @@ LAUNCHERS = ["embedding", "rmsnorm", "layernorm", "scale_", "rope_table", "rope_
              "attention_prefill_bf16", "attention_decode_bf16", "pwa_prepare", "pwa_pool", "pwa_attend", "pwa_prefill_bf16", "pwa_decode_bf16",
              "glr_scan", "glr_scan_pieces", "head_rmsnorm", "argmax", "wkv_scan", "wkv_scan_pieces", "shift_mix", "head_norm_gate", "tanh",
              "latent_prepare", "head_linear", "route_topk", "experts_up", "experts_down", "experts_sort", "experts_gather",
-             "experts_combine", "experts_up_grouped", "experts_down_grouped", "clamped_glu", "add_bias_rows"]
+             "experts_combine", "experts_up_grouped", "experts_down_grouped", "experts_gemm", "clamped_glu", "add_bias_rows"]
 
 
 def kernel_share(torch, eng, entries_of, classes):

@@ -344,3 +344,119 @@ extern "C" int br_experts_down_grouped(const void* y, const void* w_down, const 
     experts_down_grouped_kernel<<<dim3(E, (W + 31) / 32), 256, 0, s>>>((const bf16*)y, (const bf16*)w_down, first, out, W, F);
     return br_check_launch();
 }
+
+// ------------------------------------------- many tokens, all experts in one launch -----
+// C[p, :] = W[e] A[p, :] for the pairs p of every expert e in the experts' order (A's rows lie in that order).
+// bfloat16 on the matrix cores: a workgroup owns 128 pairs of ONE expert x 128 outputs; which expert and which of its
+// pairs follows from `first` (the workgroup's number counts the experts' tiles of 128 pairs in turn; numbers beyond
+// the last tile leave at once).  K goes 64 at a time through two LDS stages (rows 144 bytes apart so that a lane's
+// 16-byte reads spread over the banks), the next stage's rows in registers while the current one is multiplied, one
+// barrier a stage; four waves as 2 x 2, each 64 pairs x 64 outputs in four blocks of v_mfma_f32_32x32x16_bf16 with
+// the weight rows as the first operand.  grid (ceil(pairs / 128) + E, ceil(N / 128)).  K in steps of 8.
+#define RX_KT 64                   // k a stage
+#define RX_LD (RX_KT + 8)          // elements from one LDS row to the next
+template <typename OutT>
+__global__ __launch_bounds__(256, 2) void experts_gemm_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wt,
+                                                              const int* __restrict__ first, OutT* __restrict__ C, int E, int N, int K) {
+    constexpr int TPR = RX_KT / 8;             // threads that bring one row of a stage
+    constexpr int RPP = 256 / TPR;             // rows a pass of the workgroup brings
+    constexpr int NP = 128 / RPP;              // passes a tile
+    __shared__ __attribute__((aligned(16))) bf16 As[2][128][RX_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Ws[2][128][RX_LD];
+    int tile = blockIdx.x, e = 0, p0 = 0, p1 = 0;
+    bool found = false;
+    for (e = 0; e < E; ++e) {
+        const int a = first[e], b = first[e + 1], nt = (b - a + 127) >> 7;
+        if (tile < nt) { p0 = a + tile * 128; p1 = b; found = true; break; }
+        tile -= nt;
+    }
+    if (!found) return;
+    const int n0 = blockIdx.y * 128;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1, c = lane & 31, g = lane >> 5;
+    const int lr = tid / TPR, kc = (tid % TPR) * 8;
+    bool va[NP], vw[NP];
+    const bf16* ap[NP];
+    const bf16* wp[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        va[i] = p0 + lr + i * RPP < p1;
+        vw[i] = n0 + lr + i * RPP < N;
+        ap[i] = A + (size_t)(va[i] ? p0 + lr + i * RPP : p1 - 1) * K + kc;
+        wp[i] = Wt + ((size_t)e * N + (vw[i] ? n0 + lr + i * RPP : N - 1)) * K + kc;
+    }
+    bf16x8 zero;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) zero[i] = (bf16)0.f;
+    bf16x8 ra[NP], rw[NP];
+    auto fetch = [&](int k0) {
+        const bool on = k0 + kc < K;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            ra[i] = (on && va[i]) ? *(const bf16x8*)(ap[i] + k0) : zero;
+            rw[i] = (on && vw[i]) ? *(const bf16x8*)(wp[i] + k0) : zero;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            *(bf16x8*)&As[buf][lr + i * RPP][kc] = ra[i];
+            *(bf16x8*)&Ws[buf][lr + i * RPP][kc] = rw[i];
+        }
+    };
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += RX_KT) {
+        const bool more = k0 + RX_KT < K;
+        if (more) fetch(k0 + RX_KT);
+#pragma unroll
+        for (int kk = 0; kk < RX_KT / 16; ++kk) {
+            bf16x8 af[2], wf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                af[i] = *(const bf16x8*)&As[buf][wm * 64 + i * 32 + c][kk * 16 + 8 * g];
+                wf[i] = *(const bf16x8*)&Ws[buf][wn * 64 + i * 32 + c][kk * 16 + 8 * g];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int p = p0 + wm * 64 + j * 32 + c;
+        if (p >= p1) continue;
+        OutT* crow = C + (size_t)p * N;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int n = n0 + wn * 64 + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (n < N) crow[n] = from_f32<OutT>(acc[i][j][r]);
+            }
+    }
+}
+
+extern "C" int br_experts_gemm(const void* A, const void* Wt, const int* first, void* C, int out_is_bf16, int pairs, int E,
+                               int N, int K, hipStream_t s) {
+    if (pairs <= 0) return BR_OK;
+    if (E <= 0 || N <= 0 || K <= 0 || K % 8 || ((uintptr_t)A % 16) || ((uintptr_t)Wt % 16) || (N + 127) / 128 > 65535) return BR_BAD_ARG;
+    dim3 grid((pairs + 127) / 128 + E, (N + 127) / 128);
+    if (out_is_bf16) experts_gemm_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)A, (const bf16*)Wt, first, (bf16*)C, E, N, K);
+    else experts_gemm_kernel<float><<<grid, 256, 0, s>>>((const bf16*)A, (const bf16*)Wt, first, (float*)C, E, N, K);
+    return br_check_launch();
+}

@@ -973,6 +973,18 @@ def experts_down_grouped(y: torch.Tensor, w_down: torch.Tensor, first: torch.Ten
     _check(f(_ptr(y), _ptr(w_down), _ptr(first), _ptr(out), E, W, F, _stream()), "experts_down_grouped")
 
 
+def experts_gemm(a: torch.Tensor, w: torch.Tensor, first: torch.Tensor, out: torch.Tensor) -> None:
+    """out[p] = w[e] a[p] for the pairs p of every expert e in the experts' order (`experts_sort`): a [pairs, K] bfloat16
+    rows in that order, w [E, N, K] bfloat16, out [pairs, N] bfloat16 or float32; one launch for all experts."""
+    _dev("experts_gemm", a, w, first, out)
+    n, Kd = a.shape
+    E, N, _ = w.shape
+    _req(a.dtype == w.dtype == torch.bfloat16 and Kd % 8 == 0 and w.shape == (E, N, Kd) and out.shape == (n, N)
+         and first.dtype == torch.int32 and first.numel() == E + 1, "experts_gemm: bfloat16 [pairs, K] x [E, N, K], K in steps of 8")
+    f = _fn("routed_experts", "br_experts_gemm", [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P])
+    _check(f(_ptr(a), _ptr(w), _ptr(first), _ptr(out), _is_bf16(out, "experts_gemm"), n, E, N, Kd, _stream()), "experts_gemm")
+
+
 # ------------------------------------------------------------- clamped gated unit -----
 def clamped_glu(gu: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, limit: float, alpha: float) -> None:
     """out = g sigmoid(alpha g) (u + 1), g = min(gate + b, limit), u = clamp(up + b, -limit, limit), from the float sums

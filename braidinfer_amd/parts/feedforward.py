@@ -188,21 +188,28 @@ class RoutedExperts(FeedForward):
             K.experts_down_grouped(y, self.w_down, first, out)
             K.experts_combine(out, place, share, x)
             return
-        # many tokens: expert by expert through the matrix products, the experts' row counts read by the host
         rows = step.ws.get("moe_rows", (n, self.H), dt)
         K.experts_gather(h, order, rows, self.top)
-        starts = first.tolist()
         gu = step.ws.get("moe_gu", (n, 2 * self.I), dt)
         act = step.ws.get("moe_act", (n, self.I), dt)
         out = step.ws.get("moe_out", (n, self.H), torch.float32)
-        scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if dt == torch.bfloat16 else None
-        for e in range(self.E):
-            a, b = starts[e], starts[e + 1]
-            if b > a:
-                sc = scratch if 16 < b - a <= 1024 else None          # products that may be cut along k
-                K.gemm(rows[a:b], self.w_gu[e], gu[a:b], scratch=sc)
-                K.silu_mul(gu[a:b], act[a:b])
-                K.gemm(act[a:b], self.w_down[e], out[a:b], scratch=sc)
+        if K.experts_grouped_takes(dt, self.H, self.I) and os.environ.get("BRAIDINFER_EXPERTS_ONE_BY_ONE", "") != "1":
+            # many tokens: tiles of 128 pairs of one expert, all experts in one launch a product
+            K.experts_gemm(rows, self.w_gu, first, gu)
+            K.silu_mul(gu, act)
+            K.experts_gemm(act, self.w_down, first, out)
+        else:
+            # the 32-bit path and other widths: expert by expert through the library's products, the experts' row
+            # counts read by the host
+            starts = first.tolist()
+            scratch = step.ws.get("gemm_scratch", (K.GEMM_SCRATCH_FLOATS,), torch.float32) if dt == torch.bfloat16 else None
+            for e in range(self.E):
+                a, b = starts[e], starts[e + 1]
+                if b > a:
+                    sc = scratch if 16 < b - a <= 1024 else None          # products that may be cut along k
+                    K.gemm(rows[a:b], self.w_gu[e], gu[a:b], scratch=sc)
+                    K.silu_mul(gu[a:b], act[a:b])
+                    K.gemm(act[a:b], self.w_down[e], out[a:b], scratch=sc)
         K.experts_combine(out, place, share, x)
 
 

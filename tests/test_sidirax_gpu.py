@@ -329,7 +329,7 @@ def test_routing_and_experts():
     from braidinfer_amd import kernels as K
     rng = np.random.default_rng(5)
     for T, W, F, E, top, dtype in ((9, 50, 20, 7, 3, torch.float32), (4, 64, 24, 70, 5, torch.float32), (3, 32, 16, 2, 2, torch.float32),
-                                   (6, 64, 32, 8, 1, torch.bfloat16), (70, 72, 40, 5, 3, torch.bfloat16)):
+                                   (6, 64, 32, 8, 1, torch.bfloat16), (70, 72, 40, 5, 3, torch.bfloat16), (700, 136, 200, 3, 2, torch.bfloat16)):
         h = P.to_bf16(rng.standard_normal((T, W)))
         w = {"router": P.to_bf16(rng.standard_normal((E, W))), "router.b": P.to_bf16(rng.standard_normal(E))}
         w["router"][1] = w["router"][0]                       # two experts that always tie: the lower number goes first
@@ -370,6 +370,19 @@ def test_routing_and_experts():
             x2 = torch.tensor(x0).cuda()
             K.experts_combine(out, place, share, x2)
             assert np.abs(x2.cpu().numpy() - x0 - want).max() < tol * max(1.0, np.abs(want).max())
+            # and through the one launch a product for steps of many tokens
+            rows = torch.zeros((n, W), dtype=dtype, device="cuda")
+            K.experts_gather(hd, order, rows, top)
+            gu = torch.zeros((n, 2 * F), dtype=dtype, device="cuda")
+            K.experts_gemm(rows, w_gu, first, gu)
+            act = torch.zeros((n, F), dtype=dtype, device="cuda")
+            K.silu_mul(gu, act)
+            assert np.abs(act.float().cpu().numpy() - y2.float().cpu().numpy()).max() < 0.03 * float(y2.float().abs().max())
+            out3 = torch.zeros((n, W), dtype=torch.float32, device="cuda")
+            K.experts_gemm(act, stack("down"), first, out3)
+            x3 = torch.tensor(x0).cuda()
+            K.experts_combine(out3, place, share, x3)
+            assert np.abs(x3.cpu().numpy() - x0 - want).max() < 1.5 * tol * max(1.0, np.abs(want).max())
 
 
 def test_experts_in_their_order():
