@@ -544,23 +544,52 @@ extern "C" int br_wkv_scan_pieces(const float* rows, const float* w0, const floa
 // differences are float; out has the rows' type.  A sequence that brings one token also leaves its row in the
 // slot here; longer ones by `shift_keep_kernel` behind this one (their first token reads what the last replaces).
 // grid (T, ceil(W / 256)).
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void shift_mix_kernel(const T* __restrict__ h, const float* __restrict__ mu,
                                                         T* __restrict__ out, float* __restrict__ kept, size_t slot_stride,
                                                         const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
                                                         const int* __restrict__ slots, int n_tok, int W, int n_mix) {
-    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    // a thread brings V neighbouring columns (16 bytes of a row where the width allows it)
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    const int t = blockIdx.x, i = (blockIdx.y * 256 + threadIdx.x) * V;
     if (i >= W) return;
     const int b = seq_of_token[t], slot = slots[b];
     const int t0 = cu_seqlens[b], t1 = cu_seqlens[b + 1];
-    const float cur = to_f32<T>(h[(size_t)t * W + i]);
-    float prev = 0.f;
-    if (t > t0) prev = to_f32<T>(h[(size_t)(t - 1) * W + i]);
-    else if (slot >= 0) prev = kept[(size_t)slot * slot_stride + i];
-    const float diff = prev - cur;
-    for (int s = 0; s < n_mix; ++s)
-        out[((size_t)s * n_tok + t) * W + i] = from_f32<T>(fmaf(diff, mu[(size_t)s * W + i], cur));
-    if (slot >= 0 && t1 - t0 == 1) kept[(size_t)slot * slot_stride + i] = cur;
+    float cur[V], diff[V];
+    if (V > 1) {
+        const vec_t c = *(const vec_t*)(h + (size_t)t * W + i);
+#pragma unroll
+        for (int x = 0; x < V; ++x) cur[x] = to_f32<T>(c[x]);
+    } else {
+        cur[0] = to_f32<T>(h[(size_t)t * W + i]);
+    }
+    if (t > t0) {
+        if (V > 1) {
+            const vec_t p = *(const vec_t*)(h + (size_t)(t - 1) * W + i);
+#pragma unroll
+            for (int x = 0; x < V; ++x) diff[x] = to_f32<T>(p[x]) - cur[x];
+        } else {
+            diff[0] = to_f32<T>(h[(size_t)(t - 1) * W + i]) - cur[0];
+        }
+    } else {
+#pragma unroll
+        for (int x = 0; x < V; ++x) diff[x] = (slot >= 0 ? kept[(size_t)slot * slot_stride + i + x] : 0.f) - cur[x];
+    }
+    for (int s = 0; s < n_mix; ++s) {
+        T* o = out + ((size_t)s * n_tok + t) * W + i;
+        if (V > 1) {
+            vec_t r;
+#pragma unroll
+            for (int x = 0; x < V; ++x) r[x] = from_f32<T>(fmaf(diff[x], mu[(size_t)s * W + i + x], cur[x]));
+            *(vec_t*)o = r;
+        } else {
+            o[0] = from_f32<T>(fmaf(diff[0], mu[(size_t)s * W + i], cur[0]));
+        }
+    }
+    if (slot >= 0 && t1 - t0 == 1) {
+#pragma unroll
+        for (int x = 0; x < V; ++x) kept[(size_t)slot * slot_stride + i + x] = cur[x];
+    }
 }
 
 // The last row of every sequence that brought more than one token into its slot.  grid (B, ceil(W / 256)).
@@ -579,9 +608,18 @@ extern "C" int br_shift_mix(const void* h, int is_bf16, const float* mu, void* o
                             int single_tokens, hipStream_t s) {
     if (T <= 0 || B <= 0) return BR_OK;
     if (W <= 0 || n_mix <= 0 || !kept || slot_stride < (size_t)W || (W + 255) / 256 > 65535 || B > 65535) return BR_BAD_ARG;
-    dim3 grid(T, (W + 255) / 256), keep_grid(B, (W + 255) / 256);
-    if (is_bf16) shift_mix_kernel<bf16><<<grid, 256, 0, s>>>((const bf16*)h, mu, (bf16*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
-    else shift_mix_kernel<float><<<grid, 256, 0, s>>>((const float*)h, mu, (float*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+    dim3 keep_grid(B, (W + 255) / 256);
+    // 16 bytes a thread where every row starts at a multiple of 16 bytes
+    const bool vec = W % (is_bf16 ? 8 : 4) == 0 && (((uintptr_t)h | (uintptr_t)out) % 16) == 0;
+    const int v = vec ? (is_bf16 ? 8 : 4) : 1;
+    dim3 grid(T, (W / v + 255) / 256);
+    if (is_bf16) {
+        if (vec) shift_mix_kernel<bf16, 8><<<grid, 256, 0, s>>>((const bf16*)h, mu, (bf16*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+        else shift_mix_kernel<bf16, 1><<<grid, 256, 0, s>>>((const bf16*)h, mu, (bf16*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+    } else {
+        if (vec) shift_mix_kernel<float, 4><<<grid, 256, 0, s>>>((const float*)h, mu, (float*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+        else shift_mix_kernel<float, 1><<<grid, 256, 0, s>>>((const float*)h, mu, (float*)out, kept, slot_stride, seq_of_token, cu_seqlens, slots, T, W, n_mix);
+    }
     int rc = br_check_launch();
     if (rc != BR_OK || single_tokens) return rc;
     if (is_bf16) shift_keep_kernel<bf16><<<keep_grid, 256, 0, s>>>((const bf16*)h, kept, slot_stride, cu_seqlens, slots, W);

@@ -634,7 +634,7 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const int* __restrict__ slots,
     const int* __restrict__ ctx_lens, const int* __restrict__ block_table, int table_stride,
     const bf16* __restrict__ storage, const int* __restrict__ pooled_table, int pooled_stride,
-    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks) {
+    const bf16* __restrict__ pooled, int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, int cache_heads) {
     extern __shared__ float lds[];
     const int b = blockIdx.y, kvh = blockIdx.x;
     const int slot = slots[b];
@@ -662,8 +662,11 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
         for (int r = 0; r < 16; ++r) acc_o[i][r] = 0.f;
     float m = (sink && wave == 0) ? (sinks ? sinks[head] * PWA_LOG2E : 0.f) : -INFINITY, lsum = (sink && wave == 0 && g == 0) ? 1.f : 0.f;
     const float scale2 = scale * PWA_LOG2E;
-    const size_t page_elems = (size_t)nkv * PWA_PAGE * (dk + dv);
-    const size_t k_off = (size_t)kvh * PWA_PAGE * dk, v_off = (size_t)nkv * PWA_PAGE * dk + (size_t)kvh * dv * PWA_PAGE;
+    // `nkv` blocks of query heads over `cache_heads` kv heads of the cache (more blocks than kv heads: several
+    // workgroups read the same rows, each for its own query heads)
+    const int ckv = (int)((long long)kvh * cache_heads / nkv);
+    const size_t page_elems = (size_t)cache_heads * PWA_PAGE * (dk + dv);
+    const size_t k_off = (size_t)ckv * PWA_PAGE * dk, v_off = (size_t)cache_heads * PWA_PAGE * dk + (size_t)ckv * dv * PWA_PAGE;
     int seen = 0;
     if (pool > 0 && pq - size - pool + 1 >= 0) seen = (pq - size - pool + 1) / pool + 1;
     const int far_blocks = (seen + 31) / 32;
@@ -733,7 +736,7 @@ __global__ __launch_bounds__(64 * PWA_DW) void pwa_decode_kernel(
 template <int NBK>
 static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStream_t s, const bf16* q, bf16* out, const int* slots,
                                const int* ctx, const int* bt, int ts, const bf16* st, const int* pt, int ps, const bf16* pl,
-                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds) {
+                               int nq, int nkv, int dk, int dv, int size, int pool, float scale, int sink, const float* __restrict__ sinks, size_t head_lds, int cache_heads) {
     // merges beyond 64 KB of LDS (many query heads to a kv head with wide values) are asked for once per kernel
 #define PWA_GO(V) do { \
         auto kern = pwa_decode_kernel<NBK, V>; \
@@ -743,7 +746,7 @@ static int pwa_decode_launch_v(int nbv, dim3 grid, size_t lds_of_nbv16, hipStrea
             if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return BR_LAUNCH_FAILED; \
             have = lds; \
         } \
-        kern<<<grid, 64 * PWA_DW, lds, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks); \
+        kern<<<grid, 64 * PWA_DW, lds, s>>>(q, out, slots, ctx, bt, ts, st, pt, ps, pl, nq, nkv, dk, dv, size, pool, scale, sink, sinks, cache_heads); \
     } while (0)
     if (nbv <= 1) PWA_GO(1);
     else if (nbv <= 2) PWA_GO(2);
@@ -768,9 +771,12 @@ extern "C" int br_pwa_decode_takes(int nq, int nkv, int dk, int dv) {
 extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, const int* ctx_lens, const int* block_table,
                                   int table_stride, const void* storage, const int* pooled_table, int pooled_stride,
                                   const void* pooled, int B, int nq, int nkv, int dk, int dv, int size, int pool, float scale,
-                                  int sink, const float* __restrict__ sinks, hipStream_t s) {
+                                  int sink, const float* __restrict__ sinks, int cache_heads, hipStream_t s) {
+    // `nkv` counts the blocks of query heads a workgroup serves; the cache holds `cache_heads` kv heads (0: as many),
+    // which `nkv` is a multiple of
     if (B <= 0) return BR_OK;
-    if (!br_pwa_decode_takes(nq, nkv, dk, dv) || nkv > 65535 || B > 65535 || size <= 0 || pool < 0 ||
+    if (cache_heads <= 0) cache_heads = nkv;
+    if (!br_pwa_decode_takes(nq, nkv, dk, dv) || nkv > 65535 || B > 65535 || size <= 0 || pool < 0 || nkv % cache_heads ||
         (pool > 0 && (!pooled_table || !pooled)))
         return BR_BAD_ARG;
     const int G = nq / nkv;
@@ -778,7 +784,7 @@ extern "C" int br_pwa_decode_bf16(const void* q, void* out, const int* slots, co
     const int nbk = (dk + 31) / 32, nbv = (dv + 31) / 32;
     const size_t head_lds = (size_t)2 * PWA_DW * 2 * G * sizeof(float), per_v = (size_t)PWA_DW * 16 * 2 * G * sizeof(float);
 #define PWA_K(KK) pwa_decode_launch_v<KK>(nbv, grid, per_v, s, (const bf16*)q, (bf16*)out, slots, ctx_lens, block_table, table_stride, \
-                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, head_lds)
+                                          (const bf16*)storage, pooled_table, pooled_stride, (const bf16*)pooled, nq, nkv, dk, dv, size, pool, scale, sink, sinks, head_lds, cache_heads)
     if (nbk <= 1) return PWA_K(1);
     if (nbk <= 2) return PWA_K(2);
     if (nbk <= 3) return PWA_K(3);

@@ -647,22 +647,25 @@ def pwa_decode_takes(dtype: torch.dtype, nq: int, nkv: int, dk: int, dv: int, pa
 def pwa_decode_bf16(q: torch.Tensor, out: torch.Tensor, slots: torch.Tensor, ctx_lens: torch.Tensor, block_table: torch.Tensor,
                     unit: torch.Tensor, pooled_table: Optional[torch.Tensor], pooled: Optional[torch.Tensor], B: int, nq: int,
                     nkv: int, dk: int, dv: int, page: int, size: int, pool: int, scale: float, sink: bool,
-                    sinks: Optional[torch.Tensor] = None) -> None:
+                    sinks: Optional[torch.Tensor] = None, cache_heads: int = 0) -> None:
     """Steps of one token per sequence on the matrix cores (row b of q is sequence b's token): a workgroup per
-    (kv head, sequence) serves all query heads of the kv head."""
+    (kv head, sequence) serves all query heads of the kv head.  `cache_heads` (0: nkv): the kv heads the cache holds
+    when `nkv` is a multiple of them: the query heads of one cache head are then dealt to several workgroups (many
+    query heads over one row a token, whose merge would not fit one workgroup's LDS)."""
     _dev("pwa_decode_bf16", q, out, slots, ctx_lens, block_table, unit, pooled_table, pooled)
-    _req(pwa_decode_takes(q.dtype, nq, nkv, dk, dv, page), "pwa_decode_bf16: sizes outside what the kernel takes")
+    held = cache_heads or nkv
+    _req(pwa_decode_takes(q.dtype, nq, nkv, dk, dv, page) and nkv % held == 0, "pwa_decode_bf16: sizes outside what the kernel takes")
     _req(q.shape == (B, nq * dk) and out.shape == (B, nq * dv) and out.dtype == unit.dtype == torch.bfloat16,
          "pwa_decode_bf16: q [B, nq*dk], out [B, nq*dv], bfloat16 like the cache")
     _req(slots.numel() >= B and ctx_lens.numel() >= B, "pwa_decode_bf16: arrays shorter than the batch")
-    _pwa_unit("pwa_decode_bf16", unit, nkv, dk, dv, page)
+    _pwa_unit("pwa_decode_bf16", unit, held, dk, dv, page)
     if pool:
         _req(pooled is not None and pooled_table is not None and pooled.dtype == unit.dtype, "pwa_decode_bf16: pooled unit missing")
-        _pwa_unit("pwa_decode_bf16", pooled, nkv, dk, dv, page)
-    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P, _P])
+        _pwa_unit("pwa_decode_bf16", pooled, held, dk, dv, page)
+    f = _fn("pooled_attention", "br_pwa_decode_bf16", [_P, _P, _P, _P, _P, c_int, _P, _P, c_int, _P] + [c_int] * 7 + [c_float, c_int, _P, c_int, _P])
     _check(f(_ptr(q), _ptr(out), _ptr(slots), _ptr(ctx_lens), _ptr(block_table), block_table.shape[1], _ptr(unit), _ptr(pooled_table),
              pooled_table.shape[1] if pooled_table is not None else 0, _ptr(pooled), B, nq, nkv, dk, dv, int(size), int(pool),
-             float(scale), int(sink), _sinks("pwa_decode_bf16", sinks, nq), _stream()), "pwa_decode_bf16")
+             float(scale), int(sink), _sinks("pwa_decode_bf16", sinks, nq), int(held), _stream()), "pwa_decode_bf16")
 
 
 # ------------------------------------------------------ gated linear recurrence -----

@@ -64,6 +64,7 @@ class LatentAttention(Mixer):
         self.q_norm_w = self.c_norm_w = self.sinks = None
         self.rot = 0
         self.force_simple = False          # tests set it to run the float kernel in bfloat16 too
+        self._blocks = {}
 
     # ---- weights -----------------------------------------------------------------------
     def weight_specs(self, prefix: str) -> List[TensorSpec]:
@@ -154,9 +155,11 @@ class LatentAttention(Mixer):
         if not step.is_decode and not self.force_simple and K.pwa_prefill_takes(dt, wide, r, ctx.page_tokens):
             K.pwa_prefill_bf16(q_wide, o_lat, step.cu_seqlens, step.slots, step.ctx_lens, ctx.block_table, unit, None, None,
                                step.n_seqs, step.max_new, nh, 1, wide, r, ctx.page_tokens, NO_WINDOW, 0, self.scale, self.sink, sinks)
-        elif step.is_decode and not self.force_simple and K.pwa_decode_takes(dt, nh, 1, wide, r, ctx.page_tokens):
+        elif step.is_decode and not self.force_simple and self._decode_blocks(dt, ctx.page_tokens):
+            # all heads read the one row a token: dealt to as few workgroups a sequence as the kernel's merge allows
             K.pwa_decode_bf16(q_wide, o_lat, step.slots, step.ctx_lens, ctx.block_table, unit, None, None, step.n_seqs,
-                              nh, 1, wide, r, ctx.page_tokens, NO_WINDOW, 0, self.scale, self.sink, sinks)
+                              nh, self._decode_blocks(dt, ctx.page_tokens), wide, r, ctx.page_tokens, NO_WINDOW, 0, self.scale,
+                              self.sink, sinks, cache_heads=1)
         else:
             K.pwa_attend(q_wide, o_lat, step.positions, step.seq_of_token, step.slots, ctx.block_table, unit, None, None,
                          nh, 1, wide, r, ctx.page_tokens, NO_WINDOW, 0, self.scale, self.sink, sinks)
@@ -164,6 +167,14 @@ class LatentAttention(Mixer):
         o = step.ws.get("la_o", (T, nh * e), dt)
         K.head_linear(o_lat.view(T, nh, r), self.w_uv, o.view(T, nh, e))
         linear(o, self.w_o, x, step.ws, accumulate=True)
+
+    def _decode_blocks(self, dt, page: int) -> int:
+        """Into how many blocks of heads the single-token kernel takes this mixer's heads (0: it does not)."""
+        key = (dt, page)
+        if key not in self._blocks:
+            self._blocks[key] = next((b for b in range(1, self.nh + 1)
+                                      if self.nh % b == 0 and K.pwa_decode_takes(dt, self.nh, b, self.r + self.dr, self.r, page)), 0)
+        return self._blocks[key]
 
     @staticmethod
     def _unit(ctx: MixerContext) -> torch.Tensor:

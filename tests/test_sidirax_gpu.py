@@ -488,8 +488,9 @@ def latent_in_portions(q, dkv, cw, sinks, H, D, DR, R, rot, freqs, mag, scale, p
         sk = dev_f(sinks) if sinks is not None else None
         if matrix and n == 1:
             o2 = torch.empty((2, H * R), dtype=dtype, device="cuda")
-            K.pwa_decode_bf16(q_wide[:1].repeat(2, 1), o2, slots, ctx, c.table, c.unit, None, None, 2, H, 1, wide, R, 64, 1 << 30, 0, scale,
-                              sinks is not None, sk)
+            blocks = next(b for b in range(1, H + 1) if H % b == 0 and K.pwa_decode_takes(dtype, H, b, wide, R, 64))
+            K.pwa_decode_bf16(q_wide[:1].repeat(2, 1), o2, slots, ctx, c.table, c.unit, None, None, 2, H, blocks, wide, R, 64, 1 << 30, 0, scale,
+                              sinks is not None, sk, cache_heads=1)
             o = o2[1:]
         elif matrix:
             K.pwa_prefill_bf16(q_wide, o, cu, slots, ctx, c.table, c.unit, None, None, 2, n, H, 1, wide, R, 64, 1 << 30, 0, scale,
@@ -517,7 +518,7 @@ def plain_latent(q, dkv, cw, sinks, H, D, DR, R, freqs, mag, scale, absorb):
 
 
 @pytest.mark.parametrize("H,D,DR,R,rot", [(4, 16, 8, 24, 8), (1, 10, 6, 14, 6), (3, 12, 4, 10, 2), (2, 8, 16, 40, 16), (2, 5, 0, 8, 0),
-                                          (16, 8, 32, 160, 32)])
+                                          (16, 8, 32, 160, 32), (48, 4, 8, 64, 8), (32, 4, 32, 224, 32)])
 def test_latent_attention_kernels(H, D, DR, R, rot):
     """prepare (norm, rotation, cache rows) and the attention kernels with a learnt sink a head, against the plain
     attention with expanded keys: whole, in portions across page borders, and token by token."""
