@@ -120,7 +120,7 @@ class ParallelResidual:
     Each half adds its output into the residual rows in its last product, the mixer first; neither reads the rows."""
 
     def first_norm(self, layer):
-        return layer.norms.get("mixer")
+        return None          # the norm's output is kept for both halves: nothing a product before could prepare in passing
 
     def run(self, layer, x, step, mixer_ctx) -> None:
         step.prepared_norm = None
