@@ -159,6 +159,7 @@ class RoutedExperts(FeedForward):
     # from this many tokens a step goes expert by expert through the matrix products (below it, every (token, slot)
     # pair reads its expert's rows itself, which is what a step of few tokens costs anyway)
     BY_EXPERT_FROM = 48
+    ONE_BY_ONE_FROM = 1536          # pairs an expert from which the experts go one by one through the library's products
 
     def forward(self, h, x, step) -> None:
         T, dt = step.n_tokens, self.rt.dtype
@@ -193,8 +194,13 @@ class RoutedExperts(FeedForward):
         gu = step.ws.get("moe_gu", (n, 2 * self.I), dt)
         act = step.ws.get("moe_act", (n, self.I), dt)
         out = step.ws.get("moe_out", (n, self.H), torch.float32)
-        if K.experts_grouped_takes(dt, self.H, self.I) and os.environ.get("BRAIDINFER_EXPERTS_ONE_BY_ONE", "") != "1":
-            # many tokens: tiles of 128 pairs of one expert, all experts in one launch a product
+        # Tiles of 128 pairs of one expert, all experts in one launch a product; from about 1,500 pairs an expert the
+        # library's own products, expert by expert, make up for their launches (8 layers of width 4,096, 32 experts,
+        # 8 chosen: 8,192 tokens 56.9 against 78.7 ms, 2,048 tokens 23.1 against 19.4; BRAIDINFER_EXPERTS_ONE_BY_ONE=0
+        # or =1 forces one, for measurements)
+        forced = os.environ.get("BRAIDINFER_EXPERTS_ONE_BY_ONE", "")
+        one_by_one = forced == "1" or (forced != "0" and n // self.E >= self.ONE_BY_ONE_FROM)
+        if K.experts_grouped_takes(dt, self.H, self.I) and not one_by_one:
             K.experts_gemm(rows, self.w_gu, first, gu)
             K.silu_mul(gu, act)
             K.experts_gemm(act, self.w_down, first, out)
