@@ -710,3 +710,47 @@ def test_presets_run(tmp_path):
     toks = tokens_of(pc, 60, 4)
     eng = B.Engine.from_folder(folder, dtype="float32", max_tokens=512)
     close(run(eng, toks, [40] + [1] * 20), P.forward(pc, pw, toks), "float32", "preset")
+
+
+def test_replay_of_given_tokens_through_the_command(folders, tmp_path):
+    """`bin/trace_run` as a child process on a Sidirax folder (one whose config.json leaves a size to a tensor): requests
+    whole, with their last tokens one by one, and two of unequal length in one batch, against the plain logits."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder, cfg, w = folders[("b", "float32")]
+    V = cfg["vocab"]
+    seqs = [tokens_of(cfg, n, 60 + n) for n in (90, 41)]
+    refs = [P.forward(cfg, w, s) for s in seqs]
+    out = str(tmp_path / "out")
+    p = subprocess.Popen([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", out,
+                          "--max-tokens", "512"], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    n = [0]
+
+    def step(entries, end=()):
+        p.stdin.write(json.dumps({"step": n[0], "entries": entries, "end": list(end)}) + "\n")
+        p.stdin.flush()
+        line = p.stdout.readline().strip()
+        assert line == f"done {n[0]}", f"trace_run said {line!r} (exit {p.poll()})"
+        path = os.path.join(out, f"{n[0]}.f32")
+        n[0] += 1
+        return np.fromfile(path, dtype="<f4").reshape(-1, V) if os.path.exists(path) else None
+
+    got = step([{"id": "w", "tokens": seqs[0], "want": [0, 63, 64, 89]}], end=["w"])
+    close(got, refs[0][[0, 63, 64, 89]], "float32", "whole")
+    assert step([{"id": "d", "tokens": seqs[0][:60], "want": []}]) is None
+    for t in range(60, 90):
+        got = step([{"id": "d", "tokens": [seqs[0][t]], "want": [0]}], end=["d"] if t == 89 else [])
+        close(got, refs[0][t:t + 1], "float32", f"one by one at {t}")
+    got = step([{"id": "a", "tokens": seqs[0][:80], "want": [79]}, {"id": "b", "tokens": seqs[1][:35], "want": [3, 34]}])
+    close(got, np.stack([refs[0][79], refs[1][3], refs[1][34]]), "float32", "a batch's prompts")
+    for t in range(6):
+        ending = ["b"] if t == 5 else []
+        got = step([{"id": "a", "tokens": [seqs[0][80 + t]], "want": [0]}, {"id": "b", "tokens": [seqs[1][35 + t]], "want": [0]}], end=ending)
+        close(got, np.stack([refs[0][80 + t], refs[1][35 + t]]), "float32", f"a batch's token {t}")
+    got = step([{"id": "a", "tokens": [seqs[0][86]], "want": [0]}], end=["a"])
+    close(got, refs[0][86:87], "float32", "the batch's longer request alone")
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
