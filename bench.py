@@ -381,7 +381,7 @@ def measure_design(torch, B, name, config, vocab, prompts, batches, context, ste
     ps = [[int(t) for t in rng.integers(0, vocab, context)] for _ in range(8)]
     eng.step([StepEntry(slots[b], ps[b], []) for b in range(8)])
     out["kernels"][f"decode_b8_ctx{context}"] = launcher_times(
-        torch, eng, lambda: eng.step([StepEntry(slots[b], [1], [0]) for b in range(8)]))
+        torch, eng, lambda: eng.step([StepEntry(slots[b], [ps[b][0]], [0]) for b in range(8)]))      # a token of its own each: experts are chosen by token
     for sl in slots:
         eng.free_slot(sl)
     del eng, sampler
